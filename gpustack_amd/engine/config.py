@@ -68,7 +68,16 @@ class PagedMixerSpec:
     * qk_norm_full: weighted RMS norm over the whole q (and k) projection,
       before rotation.
     * tied_values: no value projection of its own; the raw key projection
-      (neither normed nor rotated) serves as the value."""
+      (neither normed nor rotated) serves as the value.
+    * head_norm: weighted RMS norm of every q and k head over its own
+      channels, one weight vector of head size shared by all heads.
+    * q_temp = (coef, every): the query at position p is multiplied by
+      1 + coef * ln(floor((p + 1) / every) + 1).
+    * distance_bias: slope_h * (i - j) is taken off the scaled score of
+      query i and key j, slope_h = 2^(-8 (h + 1) / heads).
+    * v_mix: the layer's values blend with the values the FIRST such layer
+      of the stack computed for the same token, v <- (1 - l) v + l v_first
+      with one learned l per layer; the blend is what the pool keeps."""
     heads: int
     kv_heads: int
     qk_dim: int
@@ -83,6 +92,15 @@ class PagedMixerSpec:
     sink: bool = False
     qk_norm_full: bool = False
     tied_values: bool = False
+    head_norm: bool = False
+    q_temp: tuple | None = None         # (coef, every)
+    distance_bias: bool = False
+    v_mix: bool = False
+
+    def slopes(self) -> list[float]:
+        """Distance-bias slope of every head, in double precision."""
+        return [2.0 ** (-8.0 * (h + 1) / self.heads)
+                for h in range(self.heads)]
 
     @property
     def k_width(self) -> int:           # cached key channels per kv head
@@ -91,6 +109,39 @@ class PagedMixerSpec:
     @property
     def v_width(self) -> int:
         return self.qk_dim if self.tied_values else self.v_dim
+
+
+@dataclass(frozen=True)
+class ScanMixerSpec:
+    """Recurrent mixer with one matrix state per head and sequence
+    (models/state_mixers.py), S_t = a_t S_(t-1) + b_t k_t v_t^T, y_t = S_t^T
+    q_t (+ skip * v_t), the state [state x vdim] kept in fp32 in a slot of
+    the engine's state pool.
+
+    * kind "mamba2": a_t = exp(-exp(A_log) * dt_t), b_t = dt_t with dt_t =
+      softplus(dt + dt_bias) per head and token; k / q (B / C) are shared
+      by the heads of a group; v (x), B and C pass a causal convolution of
+      `conv` taps per channel and SiLU first; a per-head skip D; the output
+      is gated by silu(z), then RMS-normed in `norm_groups` parts.
+    * kind "lightning": a_t = decay[h] (constants), b_t = 1, q / k / v are
+      SiLU of their projections (one k and q per head); the output is
+      RMS-normed over all heads, then multiplied by a sigmoid gate."""
+    kind: str
+    heads: int
+    state: int                          # rows of the state = size of k and q
+    vdim: int
+    groups: int = 0                     # k/q groups (mamba2); heads otherwise
+    conv: int = 0                       # taps of the causal convolution
+    norm_groups: int = 1
+    decay: tuple | None = None
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:     # x | B | C
+        return (self.inner + 2 * self.groups * self.state) if self.conv else 0
 
 
 @dataclass(frozen=True)
@@ -112,13 +163,22 @@ class FeedForwardSpec:
     shared_ff: int = 0
     shared_gated: bool = False
     gated: bool = False
+    # routing variants: scores from a softmax over all experts or from a
+    # sigmoid per expert; a learned per-expert correction added to the
+    # scores for the CHOICE only (weights use the plain scores); a group
+    # ranked by the sum of its `group_top` best choice scores (1 = its best
+    # member); chosen scores divided by their sum before the scale
+    route_scores: str = "softmax"        # "softmax" | "sigmoid"
+    route_correction: bool = False
+    group_top: int = 1
+    renorm: bool = False
 
 
 @dataclass(frozen=True)
 class LayerSpec:
     """One entry of a heterogeneous layer stack (ModelSpec.layers)."""
-    mixer_type: str                      # "latent_attention" | "paged_attention"
-    mixer: "LatentMixerSpec | PagedMixerSpec"
+    mixer_type: str         # "latent_attention" | "paged_attention" | "scan"
+    mixer: "LatentMixerSpec | PagedMixerSpec | ScanMixerSpec"
     mlp: FeedForwardSpec | None = None
 
 
@@ -269,13 +329,34 @@ class ModelSpec:
             m = self.layers[i].mixer
             if isinstance(m, LatentMixerSpec):
                 out.append(("latent", m.kv_rank))
+            elif isinstance(m, ScanMixerSpec):
+                out.append(("state",))      # nothing per token: a state slot
             else:
                 out.append(("kv", m.kv_heads, m.k_width, m.v_width))
         return out
 
+    def state_pool_shapes(self) -> list[tuple | None]:
+        """Per layer run: None, or (heads, state, vdim, conv rows, conv
+        channels) of the recurrent state one live sequence holds there."""
+        out = []
+        for i, _ in self.layer_runs():
+            m = self.layers[i].mixer
+            if isinstance(m, ScanMixerSpec):
+                out.append((m.heads, m.state, m.vdim,
+                            max(m.conv - 1, 0), m.conv_channels))
+            else:
+                out.append(None)
+        return out
+
+    @property
+    def has_state(self) -> bool:
+        return self.layers is not None and any(
+            isinstance(ls.mixer, ScanMixerSpec) for ls in self.layers)
+
     def kv_bytes_per_token(self, dtype_size: int = 2) -> int:
         if self.layers is not None:
-            return sum(w[1] if w[0] == "latent" else w[1] * (w[2] + w[3])
+            return sum(w[1] if w[0] == "latent" else
+                       0 if w[0] == "state" else w[1] * (w[2] + w[3])
                        for w in self.kv_pool_widths()) * dtype_size
         if self.kv_lora_rank:
             # MLA: one compressed latent row per token per layer
@@ -292,12 +373,32 @@ class ModelSpec:
                 n += (self.bigram_buckets + 1) * h
             for ls in self.layers:
                 m = ls.mixer
+                if isinstance(m, ScanMixerSpec):
+                    if m.kind == "mamba2":
+                        n += (h * (2 * m.inner + 2 * m.groups * m.state
+                                   + m.heads)
+                              + m.conv_channels * (m.conv + 1)
+                              + 3 * m.heads + m.inner)
+                    else:
+                        n += (h * (2 * m.heads * m.state + 2 * m.inner)
+                              + m.inner)
+                    n += m.inner * h + 4 * h
+                    f = ls.mlp
+                    if f is not None and f.kind == "moe":
+                        n += f.experts * (2 * h * f.ff + h + 1)
+                        n += 2 * h * f.shared_ff
+                    elif f is not None:
+                        n += (3 if f.gated else 2) * h * f.ff
+                    continue
                 if isinstance(m, PagedMixerSpec):
                     n += (h * m.maps * m.qk_dim * (m.heads + m.kv_heads)
                           + (0 if m.tied_values else h * m.kv_heads * m.v_dim)
                           + m.heads * m.v_dim * h + 4 * h)
                     f = ls.mlp
-                    if f is not None:
+                    if f is not None and f.kind == "moe":
+                        n += f.experts * (2 * h * f.ff + h + 1)
+                        n += 2 * h * f.shared_ff
+                    elif f is not None:
                         n += (3 if f.gated else 2) * h * f.ff
                     continue
                 n += (h * m.heads * m.qk_dim + h * m.kv_rank + m.kv_rank
@@ -490,7 +591,107 @@ class ModelSpec:
         )
 
     @classmethod
+    def _from_livasun_config(cls, cfg: dict) -> "ModelSpec":
+        """Livasun checkpoints list their layers one by one; an entry names
+        its mixer — "attention" (windowed softmax attention without
+        rotation: per-head q/k norm, query temperature, distance bias,
+        values blended with the first such layer's), "mamba2" or
+        "lightning" (recurrent matrix states) — and its feed-forward:
+        gated dense, a routed expert bank with an always-on shared expert,
+        or none. Layers are pre-norm with layer norms (weight and bias) on
+        an fp32 stream; embeddings are scaled."""
+        layers = []
+        for ent in cfg["layers"]:
+            m, kind = ent["mixer"], ent["type"]
+            if kind == "attention":
+                mask = m.get("mask") or {}
+                qt = m.get("q_temp") or None
+                mixer = PagedMixerSpec(
+                    heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
+                    qk_dim=int(m["dim"]), v_dim=int(m.get("vdim", m["dim"])),
+                    scale=float(m["scale"]),
+                    window=int(mask.get("size", 0) or 0), head_norm=True,
+                    q_temp=(float(qt["coef"]), int(qt["every"]))
+                    if qt else None,
+                    distance_bias=True, v_mix=bool(m.get("v_mix", False)))
+                if mixer.heads % mixer.kv_heads:
+                    raise ValueError("heads must be a multiple of kv_heads")
+                if mixer.q_temp is not None and mixer.q_temp[1] < 1:
+                    raise ValueError("q_temp.every must be at least 1")
+                mtype = "paged_attention"
+            elif kind == "mamba2":
+                mixer = ScanMixerSpec(
+                    kind="mamba2", heads=int(m["heads"]),
+                    state=int(m["state"]), vdim=int(m["vdim"]),
+                    groups=int(m.get("groups", 1) or 1),
+                    conv=int(m["conv"]),
+                    norm_groups=int(m.get("norm_groups", 1) or 1))
+                if mixer.heads % mixer.groups or mixer.conv < 1 \
+                        or mixer.inner % mixer.norm_groups:
+                    raise ValueError("mamba2 sizes do not divide")
+                mtype = "scan"
+            elif kind == "lightning":
+                mixer = ScanMixerSpec(
+                    kind="lightning", heads=int(m["heads"]),
+                    state=int(m["dim"]), vdim=int(m["vdim"]),
+                    groups=int(m["heads"]),
+                    decay=tuple(float(d) for d in m["decay"]))
+                if len(mixer.decay) != mixer.heads:
+                    raise ValueError("one decay per head")
+                mtype = "scan"
+            else:
+                raise NotImplementedError(
+                    f"Livasun mixer type {kind!r} is not implemented")
+            f = ent.get("mlp")
+            if not f:
+                ff = None
+            elif f["kind"] == "dense":
+                ff = FeedForwardSpec(kind="dense", ff=int(f["ff"]),
+                                     act="silu", gated=True)
+            elif f["kind"] == "moe":
+                r = f["router"]
+                g = r.get("groups") or {}
+                sh = f.get("shared") or None
+                ff = FeedForwardSpec(
+                    kind="moe", ff=int(f["expert"]["ff"]), act="relu2",
+                    experts=int(r["experts"]), top=int(r["top"]),
+                    groups=int(g.get("count", 1) or 1),
+                    keep_groups=int(g.get("keep", g.get("count", 1)) or 1),
+                    route_scale=float(r.get("scale", 1.0)),
+                    shared_ff=int(sh["ff"]) if sh else 0,
+                    route_scores="sigmoid", route_correction=True,
+                    group_top=2, renorm=True)
+                if ff.experts % ff.groups or ff.top > ff.experts \
+                        or ff.keep_groups * (ff.experts // ff.groups) < ff.top:
+                    raise ValueError("router sizes do not fit")
+            else:
+                raise NotImplementedError(
+                    f"Livasun feed-forward kind {f['kind']!r}")
+            layers.append(LayerSpec(mtype, mixer, ff))
+        vm = [ls.mixer for ls in layers
+              if isinstance(ls.mixer, PagedMixerSpec) and ls.mixer.v_mix]
+        if any((m.kv_heads, m.v_dim) != (vm[0].kv_heads, vm[0].v_dim)
+               for m in vm):
+            raise ValueError("value-mixing layers must share a value shape")
+        return cls(
+            architecture="Livasun",
+            vocab_size=int(cfg["vocab"]),
+            hidden_size=int(cfg["width"]),
+            num_layers=len(layers),
+            layers=tuple(layers),
+            num_heads=1, num_kv_heads=1, head_dim=8, intermediate_size=0,
+            rms_norm_eps=float(cfg["norm"]["eps"]),
+            max_position_embeddings=int(
+                cfg.get("max_position_embeddings", 1 << 20)),
+            eos_token_id=int(cfg.get("eos_token_id", -1)),
+            fp32_residual=True, norm_type="layernorm_bias",
+            embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)),
+        )
+
+    @classmethod
     def from_hf_config(cls, cfg: dict) -> "ModelSpec":
+        if cfg.get("architecture") == "Livasun" and "architectures" not in cfg:
+            return cls._from_livasun_config(cfg)
         if cfg.get("architecture") == "Vunitar" and "architectures" not in cfg:
             return cls._from_vunitar_config(cfg)
         if cfg.get("architecture") == "Fusipel" and "architectures" not in cfg:

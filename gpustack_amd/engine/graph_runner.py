@@ -85,6 +85,16 @@ class DecodeGraphRunner:
             self.h_pos32 = torch.zeros(mb, dtype=torch.int32, pin_memory=pin)
             self.n_prev = self.h_prev.numpy()
             self.n_pos32 = self.h_pos32.numpy()
+        # recurrent-state models: each row's state slot; padded rows use the
+        # pool's spare slot
+        self.stateful = self.ragged and kv.state_allocator is not None
+        if self.stateful:
+            self.state_slots = torch.full((mb,), kv.pad_state_slot,
+                                          dtype=torch.int32, device=dev)
+            self.h_state_slots = torch.full((mb,), kv.pad_state_slot,
+                                            dtype=torch.int32, pin_memory=pin)
+            self.n_state_slots = self.h_state_slots.numpy()
+            self.seq_rows_one = torch.ones(mb, dtype=torch.int32, device=dev)
         self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self.outs: dict[int, torch.Tensor] = {}
         self.metas: dict[int, ForwardMeta] = {}
@@ -106,6 +116,10 @@ class DecodeGraphRunner:
                 seq_hists=[0] * bs, seq_news=[1] * bs,
                 # static launch shape: split for the longest context
                 max_ctx=self.runner.cfg.max_model_len)
+            if self.stateful:
+                meta.ragged.seq_first = self.row_seq[:bs]
+                meta.ragged.seq_rows = self.seq_rows_one[:bs]
+                meta.ragged.state_slots = self.state_slots[:bs]
         return meta
 
     def capture(self) -> None:
@@ -151,6 +165,8 @@ class DecodeGraphRunner:
                 self.n_prev[r0] = s.token_at(p0 - 1) if p0 > 0 else -1
                 for j in range(1, rps):
                     self.n_prev[r0 + j] = batch.token_ids[r0 + j - 1]
+        if self.stateful:
+            self.n_state_slots[:bs] = [s.state_slot for s in batch.seqs]
         maxb = 0
         dirty_lo, dirty_hi = self.max_bs, -1
         for si, s in enumerate(batch.seqs):
@@ -175,6 +191,8 @@ class DecodeGraphRunner:
             if self.ragged:
                 self.n_pos32[bs:hi] = 0
                 self.n_prev[bs:hi] = -1
+            if self.stateful:
+                self.n_state_slots[bs:hi] = self.runner.kv.pad_state_slot
             for i in range(bs, hi):
                 self._row_state[i] = None
             dirty_lo = min(dirty_lo, bs)
@@ -195,6 +213,9 @@ class DecodeGraphRunner:
         if self.ragged:
             self.pos32[:n].copy_(self.h_pos32[:n], non_blocking=True)
             self.prev[:n].copy_(self.h_prev[:n], non_blocking=True)
+        if self.stateful:
+            self.state_slots[:n].copy_(self.h_state_slots[:n],
+                                       non_blocking=True)
         if dirty_hi >= 0:
             self.block_tables[dirty_lo:dirty_hi + 1, :max(maxb, 1)].copy_(
                 self.h_bt[dirty_lo:dirty_hi + 1, :max(maxb, 1)], non_blocking=True

@@ -38,6 +38,31 @@ class BlockAllocator:
         self.free_list.extend(reversed(blocks))
 
 
+class StateSlotAllocator:
+    """Slots of the recurrent-state pool: a live sequence of a model with
+    recurrent mixers holds exactly one, from admission to release, whatever
+    its length. Freed slots are handed out again (last freed first); a new
+    owner starts from a zero state because its first row sits at position
+    0, not because the slot was cleared."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self.free_list: list[int] = list(range(num_slots - 1, -1, -1))
+
+    @property
+    def num_free(self) -> int:
+        return len(self.free_list)
+
+    def allocate(self) -> int:
+        if not self.free_list:
+            raise RuntimeError("out of state slots")
+        return self.free_list.pop()
+
+    def free(self, slot: int) -> None:
+        if slot >= 0:
+            self.free_list.append(slot)
+
+
 class CachingBlockAllocator(BlockAllocator):
     """Ref-counted allocator with a prefix cache (vLLM-style automatic
     prefix caching, re-designed for this engine): blocks released by a
@@ -188,7 +213,9 @@ class KVCache:
             self.num_layers = len(widths)
             self.k_caches, self.v_caches = [], []
             for w in widths:
-                if w[0] == "latent":
+                if w[0] == "state":
+                    ks = vs = (0,)
+                elif w[0] == "latent":
                     ks = (num_blocks, self.latent_planes(cfg), cfg.block_size,
                           w[1])
                     vs = (0,)
@@ -215,6 +242,40 @@ class KVCache:
             self.v_caches = [
                 torch.zeros(shape, dtype=dtype, device=device) for _ in range(self.num_layers)
             ]
+        # recurrent mixers: per layer run a matrix state [slots + 1, heads,
+        # state, vdim] in fp32 whatever the engine dtype, and the last
+        # inputs of the short convolution [slots + 1, taps - 1, channels]
+        # in the engine dtype. One slot per live sequence (max_num_seqs of
+        # them); the extra last slot takes the padded rows of a captured
+        # decode graph, as pad_block does for the paged pools
+        self.ssm_states: list = [None] * self.num_layers
+        self.conv_states: list = [None] * self.num_layers
+        self.state_allocator = None
+        self.pad_state_slot = -1
+        if self.layered and spec.has_state:
+            if getattr(cfg, "enable_prefix_caching", False):
+                raise ValueError("prefix caching cannot serve models with "
+                                 "recurrent state: a cached block holds no "
+                                 "state to resume from")
+            if getattr(cfg, "speculative", None):
+                raise ValueError("speculative decoding is not supported "
+                                 "with recurrent state (rejected drafts "
+                                 "would have advanced it)")
+            nslots = cfg.max_num_seqs
+            self.state_allocator = StateSlotAllocator(nslots)
+            self.pad_state_slot = nslots
+            act_dtype = getattr(torch, cfg.dtype)
+            for r, sh in enumerate(spec.state_pool_shapes()):
+                if sh is None:
+                    continue
+                heads, n, vdim, crows, cch = sh
+                self.ssm_states[r] = torch.zeros(
+                    (nslots + 1, heads, n, vdim), dtype=torch.float32,
+                    device=device)
+                if crows > 0:
+                    self.conv_states[r] = torch.zeros(
+                        (nslots + 1, crows, cch), dtype=act_dtype,
+                        device=device)
         # last block reserved as the graph-padding scratch block (see
         # engine/graph_runner.py): padded rows write/read there, never live KV
         self.pad_block = num_blocks - 1
@@ -314,9 +375,10 @@ class KVCache:
         if spec.layers is not None:
             esize = 4 if cfg.dtype == "float32" else 2
             planes = KVCache.latent_planes(cfg)
-            per_block = cfg.block_size * esize * sum(
-                w[1] * planes if w[0] == "latent" else w[1] * (w[2] + w[3])
-                for w in spec.kv_pool_widths())
+            per_block = max(1, cfg.block_size * esize * sum(
+                w[1] * planes if w[0] == "latent" else
+                0 if w[0] == "state" else w[1] * (w[2] + w[3])
+                for w in spec.kv_pool_widths()))
         elif spec.kv_lora_rank:
             per_block = (nl * cfg.block_size
                          * (spec.kv_lora_rank + spec.qk_rope_head_dim)

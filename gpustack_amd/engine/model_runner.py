@@ -583,13 +583,23 @@ class ModelRunner:
         for i, s in enumerate(batch.seqs):
             bt[i, : len(s.block_table)] = torch.tensor(s.block_table,
                                                        dtype=torch.int32)
-        return RaggedMeta(
+        rg = RaggedMeta(
             block_tables=bt.to(dev),
             row_seq=torch.from_numpy(row_seq).to(dev),
             pos32=positions.to(torch.int32),
             prev_tokens=torch.from_numpy(prev).to(dev),
             seq_starts=starts, seq_hists=hists, seq_news=news,
             max_ctx=max(h + n for h, n in zip(hists, news)))
+        if self.kv is not None and self.kv.state_allocator is not None:
+            if any(s.state_slot < 0 for s in batch.seqs):
+                raise RuntimeError("a scheduled sequence holds no state slot")
+            per_seq = np.asarray(
+                [starts, news, [s.state_slot for s in batch.seqs]],
+                dtype=np.int32)
+            per_seq = torch.from_numpy(per_seq).to(dev)
+            rg.seq_first, rg.seq_rows, rg.state_slots = (
+                per_seq[0], per_seq[1], per_seq[2])
+        return rg
 
     def _meta(self, batch: ScheduledBatch) -> tuple[torch.Tensor, ForwardMeta]:
         tokens, meta = self._meta_by_kind(batch)

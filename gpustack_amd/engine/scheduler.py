@@ -350,6 +350,7 @@ class Scheduler:
                     break
                 self.waiting.popleft()
                 seq.block_table = self.kv.allocator.allocate(nblocks)
+                self._take_state_slot(seq)
                 seq.num_cached_tokens = budget
                 if getattr(self.cfg, "enable_prefix_caching", False):
                     from .kv_cache import block_hashes
@@ -378,6 +379,7 @@ class Scheduler:
                 break
             self.waiting.popleft()
             seq.block_table = self.kv.allocator.allocate(nblocks)
+            self._take_state_slot(seq)
             seq.num_cached_tokens = 0
             seq.status = SeqStatus.RUNNING
             if getattr(self.cfg, "enable_prefix_caching", False):
@@ -445,6 +447,7 @@ class Scheduler:
             need = self.kv.blocks_needed(p + n) - len(seq.block_table)
             if need > 0:
                 seq.block_table.extend(self.kv.allocator.allocate(need))
+            self._take_state_slot(seq)
             seq.status = SeqStatus.RUNNING
             base = len(toks)
             batch.seqs.append(seq)
@@ -591,3 +594,13 @@ class Scheduler:
         if seq.block_table:
             self.kv.allocator.free(seq.block_table)
             seq.block_table = []
+        if seq.state_slot >= 0 and self.kv.state_allocator is not None:
+            self.kv.state_allocator.free(seq.state_slot)
+        seq.state_slot = -1
+
+    def _take_state_slot(self, seq: Sequence) -> None:
+        """Models with recurrent mixers: a sequence holds one state slot
+        from admission to release (engine/kv_cache.py). Admission is
+        bounded by max_num_seqs, which is also the number of slots."""
+        if self.kv.state_allocator is not None and seq.state_slot < 0:
+            seq.state_slot = self.kv.state_allocator.allocate()

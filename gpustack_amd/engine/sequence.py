@@ -82,6 +82,7 @@ class Sequence:
     pending_tokens: int = 0         # async decode: sampled on device, not yet read back
     next_draft: list | None = None  # draft-model speculative window (engine/eagle.py)
     lora_slot: int = 0              # 0 = no adapter (models/lora.py LoraBank)
+    state_slot: int = -1            # recurrent-state slot (engine/kv_cache.py)
     block_hashes: list | None = None  # prefix-cache chain (engine/kv_cache.py)
     guided_sm: object | None = None   # guided-JSON machine (engine/guided.py)
     guided_consumed: int = 0          # output tokens already fed to guided_sm

@@ -5,6 +5,7 @@ from .llama import LlamaForCausalLM
 _MODEL_CLASSES = {
     "Vunitar": ("vunitar", "VunitarForCausalLM"),
     "Fusipel": ("fusipel", "FusipelForCausalLM"),
+    "Livasun": ("livasun", "LivasunForCausalLM"),
 }
 
 

@@ -9,7 +9,11 @@ with full-softmax scores and group-limited top-k — experts sit in equal
 groups of neighbours, a group is ranked by its best member, only the best
 `keep_groups` groups stay eligible — and weights the chosen experts by
 score * route_scale without renormalising. An optional shared expert runs
-for every token and is scaled by a per-token sigmoid gate.
+for every token and is scaled by a per-token sigmoid gate. Variants, all
+parameters of FeedForwardSpec (ops.route_topk): sigmoid scores, a learned
+per-expert correction that counts for the choice only, groups ranked by the
+sum of their best few choice scores, chosen weights divided by their sum,
+an ungated shared expert.
 
 Router logits, scores, the gate and the weighted sum are fp32; the router
 and gate rows are fused into one fp32 GEMM on the fp32 stream.
@@ -64,6 +68,13 @@ class RoutedFF(nn.Module):
         # rows [0, E): router; row E (when gated): the shared expert's gate
         self.router_w = mk(self.e + (1 if self.gated else 0), width,
                            dt=torch.float32)
+        self.correction = (mk(self.e, dt=torch.float32)
+                           if f.route_correction else None)
+        # the plain softmax / best-member routing keeps its own kernel
+        self.scored = (f.route_scores != "softmax" or f.route_correction
+                       or f.group_top != 1 or f.renorm)
+        if f.route_scores not in ("softmax", "sigmoid"):
+            raise ValueError(f"route_scores {f.route_scores!r}")
         self.up_w = mk(self.e, f.ff, width)
         self.down_w = mk(self.e, width, f.ff)
         if f.shared_ff:
@@ -93,12 +104,21 @@ class RoutedFF(nn.Module):
     def forward(self, h, x32):
         T, W = h.shape
         dev = h.device
-        logits = F.linear(x32, self.router_w)               # fp32 [T, E(+1)]
+        # x32 None: the router reads h itself (fp32 product of its values)
+        logits = F.linear(x32 if x32 is not None else h.float(),
+                          self.router_w)                    # fp32 [T, E(+1)]
         experts = torch.empty(T, self.top, dtype=torch.int32, device=dev)
         weights = torch.empty(T, self.top, dtype=torch.float32, device=dev)
-        ops.route_grouped_topk(experts, weights, logits, self.e,
-                               self.f.groups, self.f.keep_groups,
-                               self.f.route_scale)
+        if self.scored:
+            ops.route_topk(experts, weights, logits, self.correction, self.e,
+                           self.f.groups, self.f.keep_groups,
+                           self.f.group_top,
+                           self.f.route_scores == "sigmoid", self.f.renorm,
+                           self.f.route_scale)
+        else:
+            ops.route_grouped_topk(experts, weights, logits, self.e,
+                                   self.f.groups, self.f.keep_groups,
+                                   self.f.route_scale)
         # sort the T*top assignments by expert; each expert then owns one
         # contiguous row range of the gathered activations
         TK = T * self.top

@@ -41,6 +41,12 @@ class RaggedMeta:
     seq_news: list
     max_ctx: int = 0              # longest context (host number)
     _tiles: dict | None = None
+    # device copies of the per-sequence view, for kernels that walk a
+    # sequence's rows in order (recurrent mixers), and each sequence's slot
+    # in the recurrent-state pool (None for models without such state)
+    seq_first: torch.Tensor | None = None    # [nseq] int32 first row
+    seq_rows: torch.Tensor | None = None     # [nseq] int32 rows this step
+    state_slots: torch.Tensor | None = None  # [nseq] int32
 
     def latent_tiles(self, heads: int):
         """Workgroup tile list for ops.latent_attention, cached per head

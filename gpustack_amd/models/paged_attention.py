@@ -11,7 +11,13 @@ variants, every one a parameter of PagedMixerSpec:
 * a per-head sink logit in the softmax denominator;
 * differential scores: two score maps per head share one value stream,
   out = unit_rms(a1 - lambda * a2) * (1 - diff), lambda = exp(lq1.lk1) -
-  exp(lq2.lk2) + diff.
+  exp(lq2.lk2) + diff;
+* without rotation, positions entering through the scores instead: a
+  weighted RMS norm per q / k head (one weight vector shared by the heads),
+  a query temperature growing with the logarithm of the position, a
+  per-head slope times the distance taken off every score, and values
+  blended with those the first such layer of the stack computed for the
+  same token (ops.head_norm_store prepares q and writes the pool).
 
 Flow per step: one fused q/k/v GEMM -> ops.rotary_norm_store (norm, rotary,
 cache write, all fp32 inside) -> ops.paged_attention over the block tables
@@ -33,8 +39,20 @@ from ..engine.config import PagedMixerSpec
 
 class PagedRotaryAttention(nn.Module):
     def __init__(self, width: int, m: PagedMixerSpec, eps: float, dtype,
-                 comm=None):
+                 comm=None, v_mix_first: bool = False):
         super().__init__()
+        if m.head_norm and (m.rot.dims or m.qk_norm_full or m.tied_values
+                            or m.maps != 1 or m.bias):
+            raise NotImplementedError(
+                "per-head q/k norm is served without rotation, biases, "
+                "whole-row norms, tied values or a second score map")
+        if (m.q_temp or m.v_mix) and not m.head_norm:
+            raise NotImplementedError(
+                "query temperature and value mixing come with the per-head "
+                "norm row kernel")
+        # the first value-mixing layer of a stack lends its values to the
+        # later ones and keeps its own unmixed
+        self.v_mix_first = bool(m.v_mix and v_mix_first)
         if comm is not None and comm.tp_size > 1:
             raise NotImplementedError(
                 "paged rotary attention is not sharded for tensor "
@@ -56,6 +74,15 @@ class PagedRotaryAttention(nn.Module):
         self.q_norm = mk(self.nq, dt=f32) if m.qk_norm_full else None
         self.k_norm = mk(self.nk, dt=f32) if m.qk_norm_full else None
         self.sinks = mk(m.heads, dt=f32) if m.sink else None
+        if m.head_norm:
+            self.q_head_norm = mk(m.qk_dim, dt=f32)
+            self.k_head_norm = mk(m.qk_dim, dt=f32)
+        else:
+            self.q_head_norm = self.k_head_norm = None
+        self.v_lam = mk(1, dt=f32) if m.v_mix else None
+        self.register_buffer(
+            "slopes", torch.tensor(m.slopes(), dtype=torch.float64).to(f32)
+            if m.distance_bias else None, persistent=False)
         # rows: lq1, lk1, lq2, lk2
         self.lam_vecs = mk(4, m.qk_dim, dt=f32) if m.maps == 2 else None
         self.register_buffer(
@@ -72,19 +99,34 @@ class PagedRotaryAttention(nn.Module):
                    - math.exp(float((v[2] * v[3]).sum())) + self.m.diff)
             self.lam.fill_(lam)
 
-    def forward(self, h, meta, k_cache, v_cache):
+    def forward(self, h, meta, k_cache, v_cache, shared=None):
+        """`shared`: a dict that lives for one model step; value-mixing
+        layers pass the first layer's values through it."""
         m = self.m
         T = h.shape[0]
         rg = meta.ragged
         qkv = F.linear(h, self.qkv_w, self.qkv_b)
         q = torch.empty(T, self.nq, dtype=h.dtype, device=h.device)
-        ops.rotary_norm_store(q, qkv, self.nq, self.nk, self.q_norm,
-                              self.k_norm, self.inv_freq, rg.pos32, m.qk_dim,
-                              k_cache, v_cache, meta.slot_mapping, self.eps,
-                              m.tied_values,
-                              page_groups=rg.page_groups(k_cache.shape[2])
-                              if h.is_cuda and k_cache.shape[2] == 16
-                              else None)
+        groups = (rg.page_groups(k_cache.shape[2])
+                  if h.is_cuda and k_cache.shape[2] == 16 else None)
+        if m.head_norm:
+            v_first = None
+            if m.v_mix and not self.v_mix_first:
+                v_first = shared["v_first"]
+            coef, every = m.q_temp or (0.0, 0)
+            ops.head_norm_store(q, qkv, self.nq, self.nk, self.q_head_norm,
+                                self.k_head_norm, m.qk_dim, coef, every,
+                                rg.pos32, v_first, self.v_lam, k_cache,
+                                v_cache, meta.slot_mapping, self.eps,
+                                page_groups=groups)
+            if self.v_mix_first:
+                shared["v_first"] = qkv[:, self.nq + self.nk:]
+        else:
+            ops.rotary_norm_store(q, qkv, self.nq, self.nk, self.q_norm,
+                                  self.k_norm, self.inv_freq, rg.pos32,
+                                  m.qk_dim, k_cache, v_cache,
+                                  meta.slot_mapping, self.eps, m.tied_values,
+                                  page_groups=groups)
         A = m.heads * m.maps
         # two maps meet again in fp32 (their difference cancels digits)
         a = torch.empty(T, A, self.vw, device=h.device,
@@ -94,7 +136,7 @@ class PagedRotaryAttention(nn.Module):
             rg.row_seq, rg.pos32, m.scale, maps=m.maps, window=m.window,
             keep_first=m.keep_first, sinks=self.sinks,
             tiles=rg.attn_tiles(m.heads, m.kv_heads, m.maps) if h.is_cuda
-            else None, max_ctx=rg.max_ctx)
+            else None, max_ctx=rg.max_ctx, slopes=self.slopes)
         if m.maps == 2:
             o = torch.empty(T, m.heads * self.vw, dtype=h.dtype,
                             device=h.device)

@@ -60,9 +60,14 @@ def _layered_tensor_plan(model):
     if getattr(model, "pair_table", None) is not None:
         plan.append(("bigram", model.pair_table, same))
     plan.append(("final.norm", model.final_norm, same))
+    if getattr(model, "final_norm_b", None) is not None:
+        plan.append(("final.norm.b", model.final_norm_b, same))
     plan.append(("head", model.lm_head, same))
     for i, layer in enumerate(model.layers):
         p = f"l{i}."
+        if hasattr(layer, "mixer"):
+            plan += _prenorm_layer_plan(p, layer)
+            continue
         a = layer.attn
         if hasattr(a, "qkv_w"):
             plan += _paged_layer_plan(p, layer)
@@ -141,6 +146,75 @@ def _paged_layer_plan(p: str, layer):
     return plan
 
 
+def _routed_ff_plan(p: str, m):
+    """Plan entries of a routed expert bank (models/experts.py)."""
+    same = lambda t: t
+    plan = [(p + "mlp.router", m.router_w[:m.e], same)]
+    if getattr(m, "correction", None) is not None:
+        plan.append((p + "mlp.correction", m.correction, same))
+    for e in range(m.e):
+        plan.append((p + f"mlp.e{e}.up", m.up_w[e], same))
+        plan.append((p + f"mlp.e{e}.down", m.down_w[e], same))
+    if m.shared_up_w is not None:
+        plan.append((p + "mlp.shared.up", m.shared_up_w, same))
+        plan.append((p + "mlp.shared.down", m.shared_down_w, same))
+        if m.gated:
+            plan.append((p + "mlp.shared.sg", m.router_w[m.e:], same))
+    return plan
+
+
+def _prenorm_layer_plan(p: str, layer):
+    """Plan entries of one pre-norm layer with layer norms (weight and
+    bias) whose mixer is windowed attention without rotation or a
+    recurrent matrix-state mixer (models/livasun.py): q, k and v fuse into
+    one projection, the lightning q | k | v | g into another; norm
+    weights, the convolution, step-size and decay constants stay fp32."""
+    same = lambda t: t
+    a = layer.mixer
+    plan = [(p + "norm1", layer.norm1_w, same),
+            (p + "norm1.b", layer.norm1_b, same),
+            (p + "mix.o", a.o_w, same)]
+    if hasattr(a, "qkv_w"):
+        nq, nk = a.nq, a.nk
+        plan += [(p + "mix.q", a.qkv_w[:nq], same),
+                 (p + "mix.k", a.qkv_w[nq:nq + nk], same),
+                 (p + "mix.v", a.qkv_w[nq + nk:], same),
+                 (p + "mix.q.norm", a.q_head_norm, same),
+                 (p + "mix.k.norm", a.k_head_norm, same)]
+        if a.v_lam is not None:
+            plan.append((p + "mix.vmix", a.v_lam, lambda t: t.reshape(1)))
+    elif hasattr(a, "in_w"):
+        plan += [(p + "mix.in", a.in_w, same),
+                 (p + "mix.conv", a.conv_w, same),
+                 (p + "mix.conv.b", a.conv_b, same),
+                 (p + "mix.dt_bias", a.dt_bias, same),
+                 (p + "mix.A_log", a.a_log, same),
+                 (p + "mix.D", a.skip, same),
+                 (p + "mix.norm", a.norm, same)]
+    else:
+        n, i = a.nqk, a.m.inner
+        plan += [(p + "mix.q", a.qkvg_w[:n], same),
+                 (p + "mix.k", a.qkvg_w[n:2 * n], same),
+                 (p + "mix.v", a.qkvg_w[2 * n:2 * n + i], same),
+                 (p + "mix.g", a.qkvg_w[2 * n + i:], same),
+                 (p + "mix.norm", a.norm, same)]
+    m = layer.mlp
+    if m is None:
+        return plan
+    plan += [(p + "norm2", layer.norm2_w, same),
+             (p + "norm2.b", layer.norm2_b, same)]
+    if hasattr(m, "router_w"):
+        plan += _routed_ff_plan(p, m)
+    else:
+        plan.append((p + "mlp.down", m.down_w, same))
+        if m.gated:
+            plan += [(p + "mlp.gate", m.up_w[:m.ff], same),
+                     (p + "mlp.up", m.up_w[m.ff:], same)]
+        else:
+            plan.append((p + "mlp.up", m.up_w, same))
+    return plan
+
+
 def _random_init_layered(model, cfg: EngineConfig) -> None:
     """Random weights for a heterogeneous-stack model: projections N(0,
     1/fan_in), norm and layer-scale weights near 1 / near 0.5, so deep
@@ -150,6 +224,12 @@ def _random_init_layered(model, cfg: EngineConfig) -> None:
             leaf = name.rsplit(".", 1)[-1]
             if leaf in ("b", "sink", "lq1", "lk1", "lq2", "lk2"):
                 base, std = 0.0, 0.3     # biases, sinks, lambda vectors
+            elif leaf in ("vmix", "correction", "dt_bias", "A_log"):
+                # blend weight in (0, 1); small choice corrections; step
+                # sizes around softplus(-1); decay rates around 1
+                base, std = {"vmix": (0.3, 0.05), "correction": (0.0, 0.1),
+                             "dt_bias": (-1.0, 0.5),
+                             "A_log": (0.0, 0.5)}[leaf]
             else:
                 base, std = (0.5 if leaf in ("ls1", "ls2") else 1.0), 0.05
             t = base + _gen(tuple(dst.shape), name, cfg.seed, torch.float32,

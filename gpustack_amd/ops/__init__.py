@@ -683,12 +683,15 @@ def build_attn_tiles(seq_starts, seq_hists, seq_news, heads: int,
 def paged_attention(out, q, k_cache, v_cache, block_tables, row_seq, positions,
                     scale: float, maps: int = 1, window: int = 0,
                     keep_first: int = 0, sinks=None, tiles=None,
-                    exact: bool = False, max_ctx: int = 0) -> None:
+                    exact: bool = False, max_ctx: int = 0,
+                    slopes=None) -> None:
     """q: [T, A, D], out: [T, A, VW] (A = heads * maps score maps). On the
     GPU the MFMA kernel runs for bf16 pools of fitting sizes, the fp32
     vector-ALU kernel otherwise (always for fp32 pools, or with `exact`).
     `max_ctx` (longest context in the batch, a host number) lets a batch of
-    few tiles over long contexts split each tile's keys over workgroups."""
+    few tiles over long contexts split each tile's keys over workgroups.
+    `slopes` (fp32, per head): slope * distance is taken off every scaled
+    score."""
     k = _paged_backend(q)
     if k is not None:
         if tiles is None:
@@ -705,11 +708,11 @@ def paged_attention(out, q, k_cache, v_cache, block_tables, row_seq, positions,
                                 max(1024 // nt, min(4, 2048 // nt))))
         k.paged_attention(out, q, k_cache, v_cache, block_tables, tiles,
                           positions, scale, maps, window, keep_first, sinks,
-                          exact, nsplit)
+                          exact, nsplit, slopes)
     else:
         torch_ref.paged_attention(out, q, k_cache, v_cache, block_tables,
                                   row_seq, positions, scale, maps, window,
-                                  keep_first, sinks)
+                                  keep_first, sinks, slopes)
 
 
 def diff_combine(out, a, lam, diff: float, eps: float) -> None:
@@ -726,3 +729,115 @@ def act_and_mul(out, gu, mode: str) -> None:
         k.act_and_mul(out, gu, ACT_MODES[mode])
     else:
         torch_ref.act_and_mul(out, gu, mode)
+
+
+# --- layer-norm fp32 stream, attention without rotation, recurrent mixers ---
+# ops/csrc/lnrows32.hip and ops/csrc/state_scan.hip in `_hip_state.so`.
+
+_STATE = None
+
+
+def _load_state():
+    """Load `_hip_state.so` (layer-norm row kernels, head-norm cache write,
+    short convolution, matrix-state scan, gated norms, scored routing),
+    compiling it in-tree first when no built library is there."""
+    global _STATE
+    if _STATE is not None:
+        return _STATE
+    import importlib.util
+
+    from .build import STATE_SO_PATH, build_state
+
+    if not STATE_SO_PATH.exists():
+        build_state()
+    spec = importlib.util.spec_from_file_location(
+        "gpustack_amd.ops._hip_state", STATE_SO_PATH)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    _STATE = mod
+    return mod
+
+
+def _state_backend(t: torch.Tensor):
+    return _load_state() if t.is_cuda else None
+
+
+def embed_rows_scaled(x, tokens, embed, scale: float) -> None:
+    k = _state_backend(x)
+    if k is not None:
+        k.embed_rows_scaled(x, tokens, embed, scale)
+    else:
+        torch_ref.embed_rows_scaled(x, tokens, embed, scale)
+
+
+def add_layer_norm(x, a, w, b, eps: float, h) -> None:
+    k = _state_backend(x)
+    if k is not None:
+        k.add_layer_norm(x, a, w, b, eps, h)
+    else:
+        torch_ref.add_layer_norm(x, a, w, b, eps, h)
+
+
+def head_norm_store(q_out, qkv, nq: int, nk: int, q_w, k_w, head_dim: int,
+                    temp_coef: float, temp_every: int, pos32, v_first, lam,
+                    k_cache, v_cache, slots, eps: float,
+                    page_groups=None) -> None:
+    """`page_groups` (build_page_groups; GPU, prompts): the value rows are
+    written page by page instead of row by row."""
+    k = _state_backend(qkv)
+    if k is not None:
+        k.head_norm_store(q_out, qkv, nq, nk, q_w, k_w, head_dim, temp_coef,
+                          temp_every, pos32, v_first, lam, k_cache, v_cache,
+                          slots, eps, page_groups)
+    else:
+        torch_ref.head_norm_store(q_out, qkv, nq, nk, q_w, k_w, head_dim,
+                                  temp_coef, temp_every, pos32, v_first, lam,
+                                  k_cache, v_cache, slots, eps)
+
+
+def causal_conv_silu(out, src, col0: int, w, b, conv_state, seq_first,
+                     seq_rows, state_slots, row_seq, pos32) -> None:
+    k = _state_backend(src)
+    if k is not None:
+        k.causal_conv_silu(out, src, col0, w, b, conv_state, seq_first,
+                           seq_rows, state_slots, row_seq, pos32)
+    else:
+        torch_ref.causal_conv_silu(out, src, col0, w, b, conv_state,
+                                   seq_first, seq_rows, state_slots, pos32)
+
+
+def state_scan(y, src, col_x: int, col_b: int, col_c: int, dt_src,
+               col_dt: int, heads: int, groups: int, n_state: int, vdim: int,
+               act_silu: bool, dt_bias, a_log, skip, decay, state, seq_first,
+               seq_rows, state_slots, pos32) -> None:
+    k = _state_backend(src)
+    if k is not None:
+        k.state_scan(y, src, col_x, col_b, col_c, dt_src, col_dt, heads,
+                     groups, n_state, vdim, act_silu, dt_bias, a_log, skip,
+                     decay, state, seq_first, seq_rows, state_slots, pos32)
+    else:
+        torch_ref.state_scan(y, src, col_x, col_b, col_c, dt_src, col_dt,
+                             heads, groups, n_state, vdim, act_silu, dt_bias,
+                             a_log, skip, decay, state, seq_first, seq_rows,
+                             state_slots, pos32)
+
+
+def gated_group_norm(out, y, gate, w, groups: int, eps: float,
+                     gate_first: bool) -> None:
+    k = _state_backend(y)
+    if k is not None:
+        k.gated_group_norm(out, y, gate, w, groups, eps, gate_first)
+    else:
+        torch_ref.gated_group_norm(out, y, gate, w, groups, eps, gate_first)
+
+
+def route_topk(experts, weights, logits, correction, n_experts: int,
+               groups: int, keep: int, group_top: int, sigmoid: bool,
+               renorm: bool, scale: float) -> None:
+    k = _state_backend(logits)
+    if k is not None:
+        k.route_topk(experts, weights, logits, correction, n_experts, groups,
+                     keep, group_top, sigmoid, renorm, scale)
+    else:
+        torch_ref.route_topk(experts, weights, logits, correction, n_experts,
+                             groups, keep, group_top, sigmoid, renorm, scale)

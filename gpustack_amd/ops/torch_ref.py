@@ -9,6 +9,7 @@ logic and add real kernel tests on-device).
 from __future__ import annotations
 
 import torch
+import torch.nn.functional as F
 
 
 def rms_norm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float) -> None:
@@ -535,13 +536,16 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
                     row_seq: torch.Tensor, positions: torch.Tensor,
                     scale: float, maps: int = 1, window: int = 0,
                     keep_first: int = 0,
-                    sinks: torch.Tensor | None = None) -> None:
+                    sinks: torch.Tensor | None = None,
+                    slopes: torch.Tensor | None = None) -> None:
     """out[t, a] = softmax_j(scale * q[t, a] . k_j) . V over the visible
     keys j of row t's sequence: j <= pos(t), and with window > 0 also
     (pos(t) - j < window or j < keep_first). q: [T, A, D] with A = heads *
     maps score maps (a = head * maps + map); map m of a head reads channels
     [m*D, (m+1)*D) of its kv head's key row and all maps weight the same
-    values. sinks (per head, or None) add exp(sink) to the denominator."""
+    values. sinks (per head, or None) add exp(sink) to the denominator;
+    slopes (per head, or None) take slope * (pos(t) - j) off the scaled
+    score."""
     T, A, D = q.shape
     nb, G, BS, KW = k_cache.shape
     VW = v_cache.shape[2]
@@ -560,6 +564,8 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
             g = (a // maps) // rep
             m = a % maps
             s = (K[:, g, m * D:(m + 1) * D] @ q[t, a].float()) * scale
+            if slopes is not None:
+                s = s - slopes[a // maps].float() * (p - j).float()
             mx = s.max()
             if sinks is not None:
                 mx = torch.maximum(mx, sinks[a // maps].float())
@@ -586,3 +592,200 @@ def act_and_mul(out: torch.Tensor, gu: torch.Tensor, mode: str) -> None:
     g = gu[:, :F_].float().clone()
     act_inplace(g, mode)
     out.copy_((g * gu[:, F_:].float()).to(out.dtype))
+
+
+# --- layer-norm fp32 stream, windowed attention prep, recurrent mixers ------
+# (ops/csrc/lnrows32.hip, state_scan.hip). fp32: the stream, both norms'
+# statistics, q/k head norms, the query temperature, step sizes, decays and
+# the matrix states, whatever the GEMM dtype.
+
+def embed_rows_scaled(x: torch.Tensor, tokens: torch.Tensor,
+                      embed: torch.Tensor, scale: float) -> None:
+    x.copy_(embed[tokens].float() * scale)
+
+
+def add_layer_norm(x: torch.Tensor, a: torch.Tensor | None,
+                   w: torch.Tensor | None, b: torch.Tensor | None,
+                   eps: float, h: torch.Tensor | None) -> None:
+    """x += a (fp32 stream, in place); h = (x - mean) / sqrt(var + eps) * w
+    + b in h's dtype, var the mean squared deviation. Either half may be
+    left out (a None / w None)."""
+    if a is not None:
+        x.add_(a.float())
+    if w is not None:
+        mu = x.mean(-1, keepdim=True)
+        d = x - mu
+        var = (d * d).mean(-1, keepdim=True)
+        h.copy_((d * torch.rsqrt(var + eps) * w.float() + b.float())
+                .to(h.dtype))
+
+
+def head_norm_store(q_out: torch.Tensor, qkv: torch.Tensor, nq: int, nk: int,
+                    q_w: torch.Tensor, k_w: torch.Tensor, head_dim: int,
+                    temp_coef: float, temp_every: int, pos32: torch.Tensor,
+                    v_first: torch.Tensor | None, lam: torch.Tensor | None,
+                    k_cache: torch.Tensor, v_cache: torch.Tensor,
+                    slots: torch.Tensor, eps: float) -> None:
+    """Row kernel between a fused q/k/v projection and windowed attention
+    without rotation. Every q and k head is RMS-normed over its head_dim
+    channels with one shared weight vector each; q is then multiplied by
+    1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1) (temp_every 0:
+    off); v blends with v_first, (1 - lam) v + lam v_first, when given.
+    q -> q_out [T, nq]; k and v -> their slots of k_cache [nb, G, BS, D]
+    and of the transposed pages v_cache [nb, G, VW, BS]."""
+    T = qkv.shape[0]
+    nb, G, BS, KW = k_cache.shape
+    VW = v_cache.shape[2]
+    q = qkv[:, :nq].float().reshape(T, -1, head_dim)
+    k = qkv[:, nq:nq + nk].float().reshape(T, -1, head_dim)
+    v = qkv[:, nq + nk:].float()
+    q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_w.float()
+    k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_w.float()
+    if temp_every > 0:
+        p = pos32.to(torch.float32)
+        temp = 1.0 + temp_coef * torch.log(
+            torch.floor((p + 1.0) / float(temp_every)) + 1.0)
+        q = q * temp[:, None, None]
+    if v_first is not None:
+        lm = lam.float().reshape(())
+        v = (1.0 - lm) * v + lm * v_first.float()
+    q_out.copy_(q.reshape(T, nq).to(q_out.dtype))
+    k = k.to(k_cache.dtype).view(T, G, KW)
+    v = v.to(v_cache.dtype).view(T, G, VW)
+    ok = slots >= 0
+    blk, off = slots[ok] // BS, slots[ok] % BS
+    k_cache[blk, :, off] = k[ok]
+    v_cache[blk, :, :, off] = v[ok]
+
+
+def causal_conv_silu(out: torch.Tensor, src: torch.Tensor, col0: int,
+                     w: torch.Tensor, b: torch.Tensor,
+                     conv_state: torch.Tensor, seq_first: torch.Tensor,
+                     seq_rows: torch.Tensor, state_slots: torch.Tensor,
+                     pos32: torch.Tensor) -> None:
+    """out[t, c] = silu(b[c] + sum_k w[c, k] * in_c(t - (taps - 1 - k)))
+    per channel c of src[:, col0:col0 + C], within each sequence; inputs
+    before this step's rows come from conv_state[slot] (the sequence's last
+    taps - 1 inputs, oldest first), inputs before position 0 are zero. The
+    state then takes the last taps - 1 inputs including this step's."""
+    C, taps = w.shape
+    keep = taps - 1
+    for s in range(seq_first.numel()):
+        r0, n, slot = int(seq_first[s]), int(seq_rows[s]), int(state_slots[s])
+        hist = int(pos32[r0])
+        x = src[r0:r0 + n, col0:col0 + C].float()
+        if keep:
+            old = (conv_state[slot].float() if hist > 0
+                   else torch.zeros(keep, C, device=src.device))
+            if 0 < hist < keep:
+                old = old.clone()
+                old[:keep - hist] = 0
+            full = torch.cat([old, x], 0)
+        else:
+            full = x
+        acc = b.float()[None, :].repeat(n, 1)
+        for k in range(taps):
+            acc = acc + full[k:k + n] * w[:, k].float()[None, :]
+        out[r0:r0 + n] = (acc * torch.sigmoid(acc)).to(out.dtype)
+        if keep:
+            conv_state[slot] = full[full.shape[0] - keep:].to(conv_state.dtype)
+
+
+def state_scan(y: torch.Tensor, src: torch.Tensor, col_x: int, col_b: int,
+               col_c: int, dt_src: torch.Tensor | None, col_dt: int,
+               heads: int, groups: int, n_state: int, vdim: int,
+               act_silu: bool, dt_bias: torch.Tensor | None,
+               a_log: torch.Tensor | None, skip: torch.Tensor | None,
+               decay: torch.Tensor | None, state: torch.Tensor,
+               seq_first: torch.Tensor, seq_rows: torch.Tensor,
+               state_slots: torch.Tensor, pos32: torch.Tensor) -> None:
+    """Per sequence and head, over this step's rows in order:
+        S <- a_t S + b_t k_t v_t^T;  y_t = S^T q_t + skip * v_t
+    with S [n_state, vdim] fp32 read from state[slot] (zero when the first
+    row sits at position 0) and written back at the end. v = src[:, col_x +
+    h * vdim ...], k = src[:, col_b + g * n_state ...], q = src[:, col_c +
+    g * n_state ...] with g = h // (heads / groups), all through SiLU when
+    act_silu. With dt_src: b_t = dt = softplus(dt_src[t, col_dt + h] +
+    dt_bias[h]), a_t = exp(-exp(a_log[h]) * dt); otherwise a_t = decay[h]
+    and b_t = 1. y: [T, heads * vdim] fp32."""
+    rep = heads // groups
+
+    def act(t):
+        t = t.float()
+        return t * torch.sigmoid(t) if act_silu else t
+
+    for s in range(seq_first.numel()):
+        r0, n, slot = int(seq_first[s]), int(seq_rows[s]), int(state_slots[s])
+        hist = int(pos32[r0])
+        rows = src[r0:r0 + n]
+        v = act(rows[:, col_x:col_x + heads * vdim]).view(n, heads, vdim)
+        k = act(rows[:, col_b:col_b + groups * n_state]).view(n, groups, n_state)
+        q = act(rows[:, col_c:col_c + groups * n_state]).view(n, groups, n_state)
+        k = k.repeat_interleave(rep, 1)
+        q = q.repeat_interleave(rep, 1)
+        if dt_src is not None:
+            raw = (dt_src[r0:r0 + n, col_dt:col_dt + heads].float()
+                   + dt_bias.float())
+            # softplus without a switch-over: max(x, 0) + log1p(exp(-|x|))
+            dt = raw.clamp(min=0) + torch.log1p(torch.exp(-raw.abs()))
+            a = torch.exp(-torch.exp(a_log.float()) * dt)
+        else:
+            dt = torch.ones(n, heads, device=src.device)
+            a = decay.float()[None, :].expand(n, heads)
+        S = (state[slot].clone() if hist > 0
+             else torch.zeros_like(state[slot]))
+        for t in range(n):
+            S = a[t][:, None, None] * S + (dt[t][:, None] * k[t])[:, :, None] \
+                * v[t][:, None, :]
+            o = torch.einsum("hnp,hn->hp", S, q[t])
+            if skip is not None:
+                o = o + skip.float()[:, None] * v[t]
+            y[r0 + t] = o.reshape(-1)
+        state[slot] = S
+
+
+def gated_group_norm(out: torch.Tensor, y: torch.Tensor, gate: torch.Tensor,
+                     w: torch.Tensor, groups: int, eps: float,
+                     gate_first: bool) -> None:
+    """gate_first: u = y * silu(gate), then RMS norm of each of `groups`
+    equal parts of the row by its own root mean square, times w. Otherwise:
+    RMS norm of y in parts, times w, times sigmoid(gate). y fp32 [T, C]."""
+    T, C = y.shape
+    g = gate.float()
+    u = y * (g * torch.sigmoid(g)) if gate_first else y
+    u = u.view(T, groups, C // groups)
+    u = (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps)).view(T, C)
+    u = u * w.float()
+    if not gate_first:
+        u = u * torch.sigmoid(g)
+    out.copy_(u.to(out.dtype))
+
+
+def route_topk(experts: torch.Tensor, weights: torch.Tensor,
+               logits: torch.Tensor, correction: torch.Tensor | None,
+               n_experts: int, groups: int, keep: int, group_top: int,
+               sigmoid: bool, renorm: bool, scale: float) -> None:
+    """Scores s = sigmoid(z) or softmax(z) over logits[:, :n_experts];
+    choice scores c = s + correction. Experts sit in `groups` equal groups
+    of neighbours; a group ranks by the sum of its group_top largest choice
+    scores and only the `keep` best groups stay eligible. The top-k by
+    choice score are written with weight s (divided by the chosen scores'
+    sum + 1e-20 when renorm) * scale."""
+    T = logits.shape[0]
+    top = experts.shape[1]
+    z = logits[:, :n_experts].float()
+    s = torch.sigmoid(z) if sigmoid else torch.softmax(z, -1)
+    c = s + correction.float() if correction is not None else s
+    if groups > 1 and keep < groups:
+        per = n_experts // groups
+        cg = c.view(T, groups, per)
+        gs = torch.topk(cg, min(group_top, per), -1)[0].sum(-1)
+        gi = torch.topk(gs, keep, -1)[1]
+        gm = torch.zeros_like(gs, dtype=torch.bool).scatter_(1, gi, True)
+        c = cg.masked_fill(~gm[:, :, None], -float("inf")).reshape(T, n_experts)
+    idx = torch.topk(c, top, -1)[1]
+    wt = s.gather(1, idx)
+    if renorm:
+        wt = wt / (wt.sum(-1, keepdim=True) + 1e-20)
+    experts.copy_(idx.to(experts.dtype))
+    weights.copy_(wt * scale)

@@ -66,7 +66,7 @@ def categories_for_model(source: str, ref: str) -> list[str] | None:
                 # layer-listed checkpoints name themselves in the singular
                 arch = ((doc.get("architectures") or [None])[0]
                         or doc.get("architecture"))
-                if arch == "Vunitar" and any(
+                if arch in ("Vunitar", "Livasun") and any(
                         (ent.get("mlp") or {}).get("kind") == "moe"
                         for ent in doc.get("layers", [])):
                     return ["llm", "moe"]
