@@ -272,7 +272,7 @@ class KVCache:
                 self.ssm_states[r] = torch.zeros(
                     (nslots + 1, heads, n, vdim), dtype=torch.float32,
                     device=device)
-                if crows > 0:
+                if cch > 0:
                     self.conv_states[r] = torch.zeros(
                         (nslots + 1, crows, cch), dtype=act_dtype,
                         device=device)

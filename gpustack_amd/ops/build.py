@@ -33,6 +33,12 @@ PAGED_SO_PATH = PKG_DIR / "_hip_paged.so"
 PAGED_SOURCES = ["rowmix32.hip", "ragged_attn.hip", "resid32.hip",
                  "paged_bindings.cpp"]
 
+# layer-norm fp32-stream row kernels, head-norm cache write, scored routing
+# and the recurrent mixers (page-wise value stores come with rowmix32.hip)
+STATE_SO_PATH = PKG_DIR / "_hip_state.so"
+STATE_SOURCES = ["lnrows32.hip", "state_scan.hip", "rowmix32.hip",
+                 "state_bindings.cpp"]
+
 
 def _torch_paths():
     import torch
@@ -148,6 +154,13 @@ def build_paged(verbose: bool = False, force: bool = True) -> Path:
                         verbose, force)
 
 
+def build_state(verbose: bool = False, force: bool = True) -> Path:
+    """Compile the layer-norm stream / recurrent mixer family into
+    `_hip_state.so`."""
+    return _build_small("_hip_state", STATE_SOURCES, STATE_SO_PATH,
+                        verbose, force)
+
+
 def _build_small(ext_name: str, sources: list[str], so_path: Path,
                  verbose: bool, force: bool) -> Path:
     """Compile one small extension, its files in parallel. Objects are
@@ -197,8 +210,13 @@ if __name__ == "__main__":
     elif "--paged" in sys.argv:
         build_paged(verbose=True)
         print(f"built {PAGED_SO_PATH}")
+    elif "--state" in sys.argv:
+        build_state(verbose=True)
+        print(f"built {STATE_SO_PATH}")
     else:
         build(verbose=True, force="--force" in sys.argv)
         build_latent(verbose=True)
         build_paged(verbose=True)
-        print(f"built {SO_PATH} {LATENT_SO_PATH} {PAGED_SO_PATH}")
+        build_state(verbose=True)
+        print(f"built {SO_PATH} {LATENT_SO_PATH} {PAGED_SO_PATH} "
+              f"{STATE_SO_PATH}")

@@ -13,7 +13,7 @@ void value_page_store_launch(const void*, long, int, void*, const long*, long, c
 void diff_combine_launch(void*, const float*, const float*, float, float, long, int, int, hipStream_t);
 void act_and_mul_launch(void*, const void*, long, int, int, int, hipStream_t);
 void argmax_f32_launch(long*, const float*, int, int, hipStream_t);
-void paged_attention_launch(void*, const void*, const void*, const void*, const int*, const int*, const int*, const float*, float, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, float*, float*, hipStream_t);
+void paged_attention_launch(void*, const void*, const void*, const void*, const int*, const int*, const int*, const float*, const float*, float, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, float*, float*, hipStream_t);
 int paged_attn_max_dim();
 int paged_attn_uses_mfma(int, int, int, int);
 
@@ -164,7 +164,8 @@ void rotary_norm_store(Tensor q_out, Tensor qkv, long nq, long nk,
 void paged_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
                      Tensor block_tables, Tensor tiles, Tensor pos32,
                      double scale, long maps, long window, long keep_first,
-                     OptTensor sinks, bool exact, long nsplit) {
+                     OptTensor sinks, bool exact, long nsplit,
+                     OptTensor slopes) {
   chk(block_tables, "block_tables", at::kInt);
   chk(tiles, "tiles", at::kInt);
   chk(pos32, "pos32", at::kInt);
@@ -196,6 +197,12 @@ void paged_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
     TORCH_CHECK(sinks->numel() == H);
     sp = sinks->data_ptr<float>();
   }
+  const float* slp = nullptr;
+  if (slopes.has_value()) {
+    chk(*slopes, "slopes", at::kFloat);
+    TORCH_CHECK(slopes->numel() == H);
+    slp = slopes->data_ptr<float>();
+  }
   const bool mfma = !exact && paged_attn_uses_mfma(q_bf, BS, D, VW);
   if (!mfma) nsplit = 1;
   TORCH_CHECK(nsplit >= 1 && nsplit <= 64);
@@ -211,7 +218,7 @@ void paged_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
   }
   paged_attention_launch(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
                          v_cache.data_ptr(), block_tables.data_ptr<int>(),
-                         tiles.data_ptr<int>(), pos32.data_ptr<int>(), sp,
+                         tiles.data_ptr<int>(), pos32.data_ptr<int>(), sp, slp,
                          (float)scale, ntiles, T, A, D, VW, KW, G, BS,
                          (int)maps, H / G, (int)block_tables.size(0),
                          (int)block_tables.size(1), (int)k_cache.size(0),
@@ -266,7 +273,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("embed_rows_f32", &embed_rows_f32);
   m.def("sandwich_add_norm", &sandwich_add_norm);
   m.def("rotary_norm_store", &rotary_norm_store);
-  m.def("paged_attention", &paged_attention);
+  m.def("paged_attention", &paged_attention, py::arg("out"), py::arg("q"),
+        py::arg("k_cache"), py::arg("v_cache"), py::arg("block_tables"),
+        py::arg("tiles"), py::arg("pos32"), py::arg("scale"), py::arg("maps"),
+        py::arg("window"), py::arg("keep_first"), py::arg("sinks"),
+        py::arg("exact"), py::arg("nsplit"), py::arg("slopes") = py::none());
   m.def("paged_attention_uses_mfma", &paged_attention_uses_mfma);
   m.def("diff_combine", &diff_combine);
   m.def("act_and_mul", &act_and_mul);

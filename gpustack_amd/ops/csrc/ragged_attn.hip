@@ -8,7 +8,9 @@
 // map): map m of a head reads channels [m*D, (m+1)*D) of its kv head's key
 // row, and all maps of a head weight the same value rows — two maps per
 // head are the two halves of differential attention, combined afterwards.
-// A per-head sink logit may join the denominator (no key, no value).
+// A per-head sink logit may join the denominator (no key, no value), and a
+// per-head slope times the distance pos(t) - j may be taken off the scaled
+// score (positions without rotation).
 //
 // Pools: keys [nblocks, G, BS, KW] with KW = maps * D (rotated at write
 // time), values with every page transposed, [nblocks, G, VW, BS], so both
@@ -58,6 +60,7 @@ struct AttnArgs {
   const int* tiles;          // [ntiles, 6] row0, nrows, a0, n_a, seq, a_step
   const int* pos32;          // [T]
   const float* sinks;        // [A / maps] or null
+  const float* slopes;       // [A / maps] or null
   float scale;
   int T, A, D, VW, KW, G, BS, maps, rep;   // rep = heads / kv heads
   int nseq, maxb, nblocks, window, keep_first;
@@ -138,6 +141,7 @@ __global__ __launch_bounds__(THREADS) void paged_attn_exact_kernel(
     m_run = p.sinks[e_a[e_s] / p.maps];
     l_run = 1.f;
   }
+  const float slope = p.slopes != nullptr ? p.slopes[e_a[e_s] / p.maps] : 0.f;
   float acc[4][NJ];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -186,8 +190,9 @@ __global__ __launch_bounds__(THREADS) void paged_attn_exact_kernel(
     float mx = -INFINITY;
 #pragma unroll
     for (int u = 0; u < KT / 16; ++u) {
-      s[u] = key_visible(k0 + kk + 16 * u, my_pos, p.window, p.keep_first)
-                 ? s[u] * p.scale : -INFINITY;
+      const int j = k0 + kk + 16 * u;
+      s[u] = key_visible(j, my_pos, p.window, p.keep_first)
+                 ? s[u] * p.scale - slope * (float)(my_pos - j) : -INFINITY;
       mx = fmaxf(mx, s[u]);
     }
 #pragma unroll
@@ -308,6 +313,7 @@ __global__ __launch_bounds__(THREADS) void paged_attn_mfma_kernel(
     m_run = p.sinks[e_a[e_s] / p.maps];
     l_run = 1.f;
   }
+  const float slope = p.slopes != nullptr ? p.slopes[e_a[e_s] / p.maps] : 0.f;
   f32x4 acc[NT];
 #pragma unroll
   for (int i = 0; i < NT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -346,8 +352,11 @@ __global__ __launch_bounds__(THREADS) void paged_attn_mfma_kernel(
       float mx = -INFINITY;
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        sv[u] = key_visible(k0 + kk + 16 * u, my_pos, p.window, p.keep_first)
-                    ? Ss[e_s * MSS + kk + 16 * u] * p.scale : -INFINITY;
+        const int j = k0 + kk + 16 * u;
+        sv[u] = key_visible(j, my_pos, p.window, p.keep_first)
+                    ? Ss[e_s * MSS + kk + 16 * u] * p.scale -
+                          slope * (float)(my_pos - j)
+                    : -INFINITY;
         mx = fmaxf(mx, sv[u]);
       }
 #pragma unroll
@@ -553,7 +562,8 @@ int paged_attn_uses_mfma(int io_bf, int BS, int D, int VW) {
 void paged_attention_launch(void* out, const void* q, const void* k_cache,
                             const void* v_cache, const int* block_tables,
                             const int* tiles, const int* pos32,
-                            const float* sinks, float scale, int ntiles, int T,
+                            const float* sinks, const float* slopes,
+                            float scale, int ntiles, int T,
                             int A, int D, int VW, int KW, int G, int BS,
                             int maps, int rep, int nseq, int maxb, int nblocks,
                             int window, int keep_first, int q_bf, int out_bf,
@@ -562,7 +572,7 @@ void paged_attention_launch(void* out, const void* q, const void* k_cache,
   if (ntiles == 0) return;
   AttnArgs p;
   p.block_tables = block_tables; p.tiles = tiles; p.pos32 = pos32;
-  p.sinks = sinks; p.scale = scale; p.T = T; p.A = A; p.D = D; p.VW = VW;
+  p.sinks = sinks; p.slopes = slopes; p.scale = scale; p.T = T; p.A = A; p.D = D; p.VW = VW;
   p.KW = KW; p.G = G; p.BS = BS; p.maps = maps; p.rep = rep; p.nseq = nseq;
   p.maxb = maxb; p.nblocks = nblocks; p.window = window;
   p.keep_first = keep_first;

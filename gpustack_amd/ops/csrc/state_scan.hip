@@ -1,0 +1,381 @@
+// Recurrent mixers with one matrix state per head and sequence (gfx950).
+//
+//   S_t = a_t S_(t-1) + b_t k_t v_t^T,    y_t = S_t^T q_t + skip * v_t
+//
+// S [N x P] is fp32 and lives in the sequence's slot of a state pool
+// [slots, H, N, P]. A batch is ragged: sequence s brings rows seq_first[s]
+// .. seq_first[s] + seq_rows[s] - 1 (a prompt portion, or one decoded
+// token); its first row's position says whether the slot is read (> 0) or
+// the state starts from zero (== 0). Every kernel here walks or indexes
+// rows through that per-sequence view, so a prompt cut anywhere, a decode
+// row and a mixed batch give the same states.
+//
+//   causal_conv_silu : short causal convolution per channel + SiLU; the
+//                      inputs before this step's rows come from the slot's
+//                      last taps - 1 inputs; a second launch moves the
+//                      slot on (it must not race with the reads)
+//   state_scan       : the recurrence. A wave owns PL value channels of one
+//                      (sequence, head); the N state rows are split over
+//                      TPP lanes per channel, NR rows each, in registers.
+//                      Rows are staged CH at a time through LDS (k, q, v,
+//                      decay, step), then walked in order. Step sizes and
+//                      decays are computed here in fp32: a = exp(-exp(A_log)
+//                      * dt), b = dt = softplus(raw + bias), or constants.
+//   gated_group_norm : gate and RMS norm in equal parts of the row, in
+//                      either order
+#include "common.h"
+
+namespace {
+
+template <typename T> DEVICE_INLINE float ld(const T* p);
+template <> DEVICE_INLINE float ld<float>(const float* p) { return *p; }
+template <> DEVICE_INLINE float ld<unsigned short>(const unsigned short* p) {
+  return bf2f(*p);
+}
+template <typename T> DEVICE_INLINE void st(T* p, float v);
+template <> DEVICE_INLINE void st<float>(float* p, float v) { *p = v; }
+template <> DEVICE_INLINE void st<unsigned short>(unsigned short* p, float v) {
+  *p = f2bf(v);
+}
+
+DEVICE_INLINE float silu_f(float z) { return z / (1.0f + expf(-z)); }
+DEVICE_INLINE float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+// softplus without a switch-over: max(x, 0) + log1p(exp(-|x|))
+DEVICE_INLINE float softplus_f(float x) {
+  return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)));
+}
+
+constexpr int MAX_TAPS = 16;
+
+// grid (T, ceil(C / 256)): one lane per (row, channel).
+template <typename TS>
+__global__ __launch_bounds__(256) void causal_conv_silu_kernel(
+    TS* __restrict__ out, const TS* __restrict__ src, long ld_src, int col0,
+    int C, int taps, const float* __restrict__ w, const float* __restrict__ b,
+    const TS* __restrict__ conv_state, const int* __restrict__ seq_first,
+    const int* __restrict__ state_slots, const int* __restrict__ row_seq,
+    const int* __restrict__ pos32, int nseq, int nslots, int T) {
+  const int t = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int s = min(max(row_seq[t], 0), nseq - 1);
+  const int first = min(max(seq_first[s], 0), t);
+  const int i = t - first;                   // row index inside the portion
+  const int pos = max(pos32[t], 0);
+  const int slot = min(max(state_slots[s], 0), nslots - 1);
+  const int keep = taps - 1;
+  const TS* stp = conv_state + (long)slot * keep * C;
+  float acc = b[c];
+  for (int k = 0; k < taps; ++k) {
+    const int d = keep - k;                  // how far back this tap looks
+    float v = 0.f;
+    if (i - d >= 0)
+      v = ld(src + (long)(t - d) * ld_src + col0 + c);
+    else if (pos - d >= 0)
+      v = ld(stp + (long)(keep + i - d) * C + c);
+    acc += w[(long)c * taps + k] * v;
+  }
+  st(out + (long)t * C + c, silu_f(acc));
+}
+
+// grid (nseq, ceil(C / 256)): the slot's new last inputs, after every read
+// of the old ones (stream order).
+template <typename TS>
+__global__ __launch_bounds__(256) void conv_state_update_kernel(
+    const TS* __restrict__ src, long ld_src, int col0, int C, int taps,
+    TS* __restrict__ conv_state, const int* __restrict__ seq_first,
+    const int* __restrict__ seq_rows, const int* __restrict__ state_slots,
+    const int* __restrict__ pos32, int nslots, int T) {
+  const int s = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int first = seq_first[s], n = seq_rows[s];
+  if (first < 0 || n < 1 || first + n > T) return;
+  const int hist = max(pos32[first], 0);
+  const int slot = min(max(state_slots[s], 0), nslots - 1);
+  const int keep = taps - 1;
+  TS* stp = conv_state + (long)slot * keep * C;
+  TS fresh[MAX_TAPS];
+  for (int j = 0; j < keep; ++j) {
+    const int i = n - (keep - j);            // local row of new entry j
+    TS v = 0;
+    if (i >= 0)
+      v = src[(long)(first + i) * ld_src + col0 + c];
+    else if (hist + i >= 0)
+      v = stp[(long)(keep + i) * C + c];
+    fresh[j] = v;
+  }
+  for (int j = 0; j < keep; ++j) stp[(long)j * C + c] = fresh[j];
+}
+
+struct ScanArgs {
+  long ld_src, ld_dt;
+  int col_x, col_b, col_c, col_dt;
+  int H, G, N, P, act;
+  const float* dt_bias;    // [H] with dt
+  const float* a_log;      // [H] with dt
+  const float* skip;       // [H] or null
+  const float* decay;      // [H] without dt
+  float* state;            // [nslots, H, N, P]
+  const int* seq_first;
+  const int* seq_rows;
+  const int* state_slots;
+  const int* pos32;
+  int nslots, T;
+};
+
+constexpr int CH = 16;     // rows staged per pass
+
+// One wave per (sequence, head, block of PL = 64 / TPP value channels).
+// lane = ns * PL + pl: channel p0 + pl, state rows n = r * TPP + ns.
+template <typename TS, typename TD, int NR, int TPP>
+__global__ __launch_bounds__(64) void state_scan_kernel(
+    float* __restrict__ y, const TS* __restrict__ src,
+    const TD* __restrict__ dt_src, ScanArgs p) {
+  constexpr int PL = 64 / TPP;
+  constexpr int NP = NR * TPP;               // padded state rows
+  __shared__ float ks[CH][NP];
+  __shared__ float qs[CH][NP];
+  __shared__ float vs[CH][PL];
+  __shared__ float a_s[CH], b_s[CH];
+  const int s = blockIdx.x, h = blockIdx.y, p0 = blockIdx.z * PL;
+  const int lane = threadIdx.x;
+  const int pl = lane % PL, ns = lane / PL;
+  const int first = p.seq_first[s], n = p.seq_rows[s];
+  if (first < 0 || n < 1 || first + n > p.T) return;
+  const int slot = min(max(p.state_slots[s], 0), p.nslots - 1);
+  const int hist = p.pos32[first];
+  const int N = p.N, P = p.P;
+  const int g = h / (p.H / p.G);
+  const int pc = p0 + pl;
+  const bool live = pc < P;
+  float* sp = p.state + ((long)slot * p.H + h) * N * P;
+  float S[NR];
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    const int nn = r * TPP + ns;
+    S[r] = (hist > 0 && live && nn < N) ? sp[(long)nn * P + pc] : 0.f;
+  }
+  const float skip = p.skip != nullptr ? p.skip[h] : 0.f;
+  const float a_rate = dt_src != nullptr ? expf(p.a_log[h]) : 0.f;
+  const float dtb = dt_src != nullptr ? p.dt_bias[h] : 0.f;
+  const float a_const = dt_src == nullptr ? p.decay[h] : 0.f;
+
+  for (int c0 = 0; c0 < n; c0 += CH) {
+    const int rows = min(CH, n - c0);
+    __syncthreads();
+    for (int i = lane; i < rows * NP; i += 64) {
+      const int r = i / NP, nn = i % NP;
+      float kv = 0.f, qv = 0.f;
+      if (nn < N) {
+        const TS* rp = src + (long)(first + c0 + r) * p.ld_src;
+        kv = ld(rp + p.col_b + g * N + nn);
+        qv = ld(rp + p.col_c + g * N + nn);
+        if (p.act) { kv = silu_f(kv); qv = silu_f(qv); }
+      }
+      ks[r][nn] = kv;
+      qs[r][nn] = qv;
+    }
+    for (int i = lane; i < rows * PL; i += 64) {
+      const int r = i / PL, c = i % PL;
+      float v = 0.f;
+      if (p0 + c < P) {
+        v = ld(src + (long)(first + c0 + r) * p.ld_src + p.col_x + h * P + p0 + c);
+        if (p.act) v = silu_f(v);
+      }
+      vs[r][c] = v;
+    }
+    if (lane < rows) {
+      if (dt_src != nullptr) {
+        const float dt = softplus_f(
+            ld(dt_src + (long)(first + c0 + lane) * p.ld_dt + p.col_dt + h) + dtb);
+        a_s[lane] = expf(-a_rate * dt);
+        b_s[lane] = dt;
+      } else {
+        a_s[lane] = a_const;
+        b_s[lane] = 1.f;
+      }
+    }
+    __syncthreads();
+    for (int r = 0; r < rows; ++r) {
+      const float a = a_s[r];
+      const float v = vs[r][pl];
+      const float bv = b_s[r] * v;
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < NR; ++j) {
+        const int nn = j * TPP + ns;
+        S[j] = a * S[j] + ks[r][nn] * bv;
+        acc += S[j] * qs[r][nn];
+      }
+#pragma unroll
+      for (int m = PL; m < 64; m <<= 1) acc += __shfl_xor(acc, m, WAVE_SIZE);
+      if (ns == 0 && live)
+        y[(long)(first + c0 + r) * p.H * P + h * P + pc] = acc + skip * v;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    const int nn = r * TPP + ns;
+    if (live && nn < N) sp[(long)nn * P + pc] = S[r];
+  }
+}
+
+constexpr int ROW_THREADS = 256;
+
+DEVICE_INLINE float block_sum(float v, float* red) {
+  v = wave_reduce_sum(v);
+  const int w = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  return red[0] + red[1] + red[2] + red[3];
+}
+
+// grid (T, groups): one workgroup per (row, part). gate_first: u = y *
+// silu(gate), out = u / rms(u) * w; else out = y / rms(y) * w * sigmoid(gate).
+template <typename TG, typename TO>
+__global__ __launch_bounds__(ROW_THREADS) void gated_group_norm_kernel(
+    TO* __restrict__ out, const float* __restrict__ y,
+    const TG* __restrict__ gate, long ld_gate, const float* __restrict__ w,
+    int C, int gs, float eps, int gate_first) {
+  __shared__ float red[4];
+  const long t = blockIdx.x;
+  const int c0 = blockIdx.y * gs;
+  const float* yr = y + t * C + c0;
+  const TG* gr = gate + t * ld_gate + c0;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < gs; i += ROW_THREADS) {
+    float u = yr[i];
+    if (gate_first) u *= silu_f(ld(gr + i));
+    ss += u * u;
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)gs + eps);
+  for (int i = threadIdx.x; i < gs; i += ROW_THREADS) {
+    const float gv = ld(gr + i);
+    float u = yr[i];
+    if (gate_first) u = u * silu_f(gv) * inv * w[c0 + i];
+    else u = u * inv * w[c0 + i] * sigmoid_f(gv);
+    st(out + t * C + c0 + i, u);
+  }
+}
+
+template <typename TS, typename TD, int NR, int TPP>
+void scan_launch(float* y, const void* src, const void* dt, const ScanArgs& p,
+                 int nseq, hipStream_t s) {
+  constexpr int PL = 64 / TPP;
+  dim3 grid(nseq, p.H, (p.P + PL - 1) / PL);
+  state_scan_kernel<TS, TD, NR, TPP><<<grid, 64, 0, s>>>(
+      y, (const TS*)src, (const TD*)dt, p);
+}
+
+// Rows of the state per lane (NR) and lanes per value channel (TPP): the
+// fewest lanes per channel that keep NR <= 32, but no more channels per wave
+// than the head has.
+template <typename TS, typename TD>
+bool scan_pick(float* y, const void* src, const void* dt, const ScanArgs& p,
+               int nseq, hipStream_t s) {
+  int tpp = 1;
+  while (tpp < 8 && ((p.N + tpp - 1) / tpp > 32 || 64 / tpp > max(p.P, 8)))
+    tpp *= 2;
+  const int nr = (p.N + tpp - 1) / tpp;
+#define SCAN_CASE(NRV, TPPV)                                              \
+  if (tpp == TPPV && nr <= NRV) {                                         \
+    scan_launch<TS, TD, NRV, TPPV>(y, src, dt, p, nseq, s);               \
+    return true;                                                          \
+  }
+#define SCAN_TPP(TPPV) \
+  SCAN_CASE(4, TPPV) SCAN_CASE(8, TPPV) SCAN_CASE(16, TPPV) SCAN_CASE(32, TPPV)
+  SCAN_TPP(1) SCAN_TPP(2) SCAN_TPP(4) SCAN_TPP(8)
+#undef SCAN_TPP
+#undef SCAN_CASE
+  return false;
+}
+
+}  // namespace
+
+int state_scan_max_state() { return 8 * 32; }
+int conv_max_taps() { return MAX_TAPS; }
+
+void causal_conv_silu_launch(void* out, const void* src, long ld_src, int col0,
+                             int C, int taps, const float* w, const float* b,
+                             void* conv_state, const int* seq_first,
+                             const int* seq_rows, const int* state_slots,
+                             const int* row_seq, const int* pos32, int nseq,
+                             int nslots, int T, int bf, hipStream_t s) {
+  if (T <= 0 || nseq <= 0) return;
+  dim3 grid(T, (C + 255) / 256), sgrid(nseq, (C + 255) / 256);
+  if (bf) {
+    causal_conv_silu_kernel<unsigned short><<<grid, 256, 0, s>>>(
+        (unsigned short*)out, (const unsigned short*)src, ld_src, col0, C, taps,
+        w, b, (const unsigned short*)conv_state, seq_first, state_slots,
+        row_seq, pos32, nseq, nslots, T);
+    if (taps > 1)
+      conv_state_update_kernel<unsigned short><<<sgrid, 256, 0, s>>>(
+          (const unsigned short*)src, ld_src, col0, C, taps,
+          (unsigned short*)conv_state, seq_first, seq_rows, state_slots, pos32,
+          nslots, T);
+  } else {
+    causal_conv_silu_kernel<float><<<grid, 256, 0, s>>>(
+        (float*)out, (const float*)src, ld_src, col0, C, taps, w, b,
+        (const float*)conv_state, seq_first, state_slots, row_seq, pos32, nseq,
+        nslots, T);
+    if (taps > 1)
+      conv_state_update_kernel<float><<<sgrid, 256, 0, s>>>(
+          (const float*)src, ld_src, col0, C, taps, (float*)conv_state,
+          seq_first, seq_rows, state_slots, pos32, nslots, T);
+  }
+}
+
+// src_bf: src and dt_src are bf16 (else fp32). Returns 0 when no
+// instantiation covers the sizes.
+int state_scan_launch(float* y, const void* src, long ld_src, int col_x,
+                      int col_b, int col_c, const void* dt_src, long ld_dt,
+                      int col_dt, int H, int G, int N, int P, int act,
+                      const float* dt_bias, const float* a_log,
+                      const float* skip, const float* decay, float* state,
+                      const int* seq_first, const int* seq_rows,
+                      const int* state_slots, const int* pos32, int nseq,
+                      int nslots, int T, int src_bf, hipStream_t s) {
+  if (T <= 0 || nseq <= 0) return 1;
+  ScanArgs p;
+  p.ld_src = ld_src; p.ld_dt = ld_dt; p.col_x = col_x; p.col_b = col_b;
+  p.col_c = col_c; p.col_dt = col_dt; p.H = H; p.G = G; p.N = N; p.P = P;
+  p.act = act; p.dt_bias = dt_bias; p.a_log = a_log; p.skip = skip;
+  p.decay = decay; p.state = state; p.seq_first = seq_first;
+  p.seq_rows = seq_rows; p.state_slots = state_slots; p.pos32 = pos32;
+  p.nslots = nslots; p.T = T;
+  if (src_bf)
+    return scan_pick<unsigned short, unsigned short>(y, src, dt_src, p, nseq, s);
+  return scan_pick<float, float>(y, src, dt_src, p, nseq, s);
+}
+
+void gated_group_norm_launch(void* out, const float* y, const void* gate,
+                             long ld_gate, const float* w, int T, int C,
+                             int groups, float eps, int gate_first, int gate_bf,
+                             int out_bf, hipStream_t s) {
+  if (T <= 0) return;
+  dim3 grid(T, groups);
+  const int gs = C / groups;
+  if (gate_bf) {
+    if (out_bf)
+      gated_group_norm_kernel<unsigned short, unsigned short>
+          <<<grid, ROW_THREADS, 0, s>>>((unsigned short*)out, y,
+                                        (const unsigned short*)gate, ld_gate, w,
+                                        C, gs, eps, gate_first);
+    else
+      gated_group_norm_kernel<unsigned short, float><<<grid, ROW_THREADS, 0, s>>>(
+          (float*)out, y, (const unsigned short*)gate, ld_gate, w, C, gs, eps,
+          gate_first);
+  } else {
+    if (out_bf)
+      gated_group_norm_kernel<float, unsigned short><<<grid, ROW_THREADS, 0, s>>>(
+          (unsigned short*)out, y, (const float*)gate, ld_gate, w, C, gs, eps,
+          gate_first);
+    else
+      gated_group_norm_kernel<float, float><<<grid, ROW_THREADS, 0, s>>>(
+          (float*)out, y, (const float*)gate, ld_gate, w, C, gs, eps,
+          gate_first);
+  }
+}
