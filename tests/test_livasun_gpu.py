@@ -98,7 +98,8 @@ def test_bf16_engine_with_block_and_slot_reuse(tmp_path, gpu_engine, name):
         reqs = {i: tf.tokens_for(cfg, n, 80 + n + rnd) for i, n in REQS.items()}
         got = tf.replay(eng, reqs, STEPS)
         for i, t in reqs.items():
-            assert tf.err(got[i], oracle.forward(cfg, w, t)) < 0.15, (rnd, i)
+            assert tl.rows_over(got[i], oracle.forward(cfg, w, t), 0.15) \
+                <= 0.1, (rnd, i)
         assert kv.state_allocator.num_free == 4
 
 
@@ -112,8 +113,8 @@ def test_bf16_logits_do_not_depend_on_the_schedule(tmp_path, gpu_engine):
         ref = oracle.forward(cfg, w, t)
         # both are rounding away from the oracle, and no further from each
         # other than from it
-        assert tf.err(mixed[i], whole.double()) < 0.15, i
-        assert tf.err(whole, ref) < 0.15, i
+        assert tl.rows_over(mixed[i], whole.double(), 0.15) <= 0.1, i
+        assert tl.rows_over(whole, ref, 0.15) <= 0.1, i
 
 
 @pytest.mark.parametrize("sizes", [[2] * 20, [3, 2, 5, 2, 16, 1, 1, 17, 2, 11],
@@ -171,10 +172,19 @@ def test_wide_states(tmp_path, gpu_engine, layers):
     assert tf.err(got, oracle.forward(cfg, w, toks)) < 5e-4
 
 
-def test_generation_with_decode_graphs(tmp_path, gpu_engine):
-    cfg, w, d = _model(tmp_path, ALIGNED)
+@pytest.mark.parametrize("routed", [False, True])
+def test_generation_with_decode_graphs(tmp_path, gpu_engine, routed):
+    """fp32 greedy decoding equals the oracle's token for token. Without
+    routed layers every decode step is a captured graph (state slots and
+    block tables in static buffers); an fp32 expert bank waits for the host
+    and decodes eagerly."""
+    kw = dict(ALIGNED)
+    if not routed:
+        kw["layers"] = [dict(L, mlp=oracle.dense(40) if (L["mlp"] or {}).get(
+            "kind") == "moe" else L["mlp"]) for L in ALIGNED["layers"]]
+    cfg, w, d = _model(tmp_path, kw)
     eng = gpu_engine(d)
-    assert eng.runner.graph_runner is not None
+    assert (eng.runner.graph_runner is not None) == (not routed)
     prompts = [tf.tokens_for(cfg, n, 40 + n) for n in (3, 70, 9)]
     outs = eng.generate(prompts, SamplingParams(max_tokens=40, temperature=0.0,
                                                 ignore_eos=True))
@@ -196,4 +206,4 @@ def test_bf16_generation_runs_and_stays_close(tmp_path, gpu_engine):
     assert len(out) == 24
     full = prompt + out
     got = tf.replay(eng, {"z": full}, [[("z", len(full))]])["z"]
-    assert tf.err(got, oracle.forward(cfg, w, full)) < 0.15
+    assert tl.rows_over(got, oracle.forward(cfg, w, full), 0.15) <= 0.1
