@@ -62,7 +62,7 @@ def parse_args():
                          "stack (prefill/decode tok/s + per-kernel roofline "
                          "shares; gpustack_amd/bench/layer_bench.py)")
     ap.add_argument("--layer-family", default="vunitar",
-                    choices=["vunitar", "fusipel"],
+                    choices=["vunitar", "fusipel", "livasun"],
                     help="model family measured by --layer-bench")
     ap.add_argument("--layer-sizes", default="small,medium",
                     help="comma list of small,medium,large for --layer-bench")

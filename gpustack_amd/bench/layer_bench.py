@@ -1,4 +1,4 @@
-"""Layer-level comparison bench: a Vunitar or Fusipel stack (`family`) at
+"""Layer-level comparison bench: a Vunitar, Fusipel or Livasun stack (`family`) at
 real-model layer sizes beside the closest llama-lineage stack of equal
 width, depth and heads (random weights, synthetic tokens). Reports end-to-end prefill and decode
 throughput through LLMEngine for both, and per-kernel rates of the new
@@ -77,6 +77,46 @@ def fusipel_spec(s, moe: bool = False):
         num_heads=1, num_kv_heads=1, head_dim=8, intermediate_size=0,
         rms_norm_eps=1e-6, max_position_embeddings=1 << 20, eos_token_id=-1,
         sandwich_norms=True, fp32_residual=True, residual_multiplier=0.7)
+
+
+def livasun_spec(s, moe: bool = False):
+    """Layers cycle windowed attention (head size 128, heads/4 kv heads,
+    window 1024, query temperature, value blend), a mamba2 mixer (inner =
+    2 x width in heads of 64, state 128, 8 groups, 4 taps), attention again
+    and a lightning mixer (heads x 128 x 128); gated SiLU feed-forward of
+    the llama stack's width, or a sigmoid-routed expert bank with a shared
+    expert."""
+    from ..engine.config import (FeedForwardSpec, LayerSpec, ModelSpec,
+                                 PagedMixerSpec, ScanMixerSpec)
+
+    H, W = s["heads"], s["width"]
+    attn = PagedMixerSpec(heads=H, kv_heads=max(1, H // 4), qk_dim=128,
+                          v_dim=128, scale=128 ** -0.5, window=1024,
+                          head_norm=True, q_temp=(0.1, 1024),
+                          distance_bias=True, v_mix=True)
+    mamba = ScanMixerSpec(kind="mamba2", heads=2 * W // 64, state=128, vdim=64,
+                          groups=8, conv=4, norm_groups=8)
+    light = ScanMixerSpec(kind="lightning", heads=H, state=128, vdim=128,
+                          groups=H, decay=tuple(
+                              1.0 - 2.0 ** (-5.0 - 5.0 * h / max(H - 1, 1))
+                              for h in range(H)))
+    if moe:
+        ff = FeedForwardSpec(kind="moe", ff=s["eff"], act="relu2",
+                             experts=s["experts"], top=4, groups=4,
+                             keep_groups=2, route_scale=2.0,
+                             shared_ff=s["eff"], route_scores="sigmoid",
+                             route_correction=True, group_top=2, renorm=True)
+    else:
+        ff = FeedForwardSpec(kind="dense", ff=s["ff"], act="silu", gated=True)
+    cycle = [("paged_attention", attn), ("scan", mamba),
+             ("paged_attention", attn), ("scan", light)]
+    return ModelSpec(
+        architecture="Livasun", vocab_size=32000, hidden_size=W,
+        num_layers=s["layers"],
+        layers=tuple(LayerSpec(*cycle[i % 4], ff) for i in range(s["layers"])),
+        num_heads=1, num_kv_heads=1, head_dim=8, intermediate_size=0,
+        rms_norm_eps=1e-5, max_position_embeddings=1 << 20, eos_token_id=-1,
+        fp32_residual=True, norm_type="layernorm_bias", embed_scale=4.0)
 
 
 def llama_spec(s, moe: bool):
@@ -431,17 +471,225 @@ def fusipel_kernel_rates(s, device):
     return out
 
 
+PEAK_VALU = 157.3e12     # fp32 vector ALU
+
+
+def livasun_kernel_rates(s, device):
+    """Per-kernel rates of the Livasun kernels next to the llama graph's
+    counterparts (the recurrent mixers have none there: their like is the
+    attention kernel of the same phase)."""
+    from .. import ops
+
+    bf = torch.bfloat16
+    H, W, D, BS = s["heads"], s["width"], 128, 16
+    G = max(1, H // 4)
+    out = []
+
+    def rec(name, sec, flops=None, nbytes=None, peak=PEAK_FLOPS):
+        if flops is not None:
+            out.append(dict(kernel=name, us=round(sec * 1e6, 1),
+                            tflops=round(flops / sec / 1e12, 1),
+                            roofline=round(flops / sec / peak, 4)))
+        else:
+            out.append(dict(kernel=name, us=round(sec * 1e6, 1),
+                            gbps=round(nbytes / sec / 1e9, 1),
+                            roofline=round(nbytes / sec / PEAK_BW, 4)))
+
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=device)
+    # ---- prefill attention: 4 prompts x 2048, window 1024 ----
+    nseq, L, win = 4, 2048, 1024
+    T = nseq * L
+    nblk = T // BS + 1
+    bt = torch.arange(nseq * (L // BS), dtype=torch.int32, device=device).view(nseq, -1)
+    row_seq = torch.arange(nseq, dtype=torch.int32, device=device).repeat_interleave(L)
+    pos = torch.arange(L, dtype=torch.int32, device=device).repeat(nseq)
+    starts = [i * L for i in range(nseq)]
+    kc = torch.randn(nblk, G, BS, D, device=device).to(bf)
+    vc = torch.randn(nblk, G, D, BS, device=device).to(bf)
+    q = torch.randn(T, H, D, device=device).to(bf)
+    o = torch.empty_like(q)
+    slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / H) for h in range(H)],
+                          device=device)
+    tiles = ops.build_attn_tiles(starts, [0] * nseq, [L] * nseq, H, G, 1, device)
+    wpairs = nseq * sum(min(i + 1, win) for i in range(L))
+    rec("paged_attention prefill, window 1024 + slopes (mfma, useful pairs)",
+        _time(lambda: ops.paged_attention(o, q, kc, vc, bt, row_seq, pos,
+                                          D ** -0.5, window=win, tiles=tiles,
+                                          slopes=slopes), 5),
+        flops=4.0 * D * H * wpairs)
+    kf = torch.randn(T, G, D, device=device).to(bf)
+    vf = torch.randn_like(kf)
+    ptiles = ops.build_prefill_tiles([L] * nseq, device)
+    rec("flash_prefill (llama graph, causal)",
+        _time(lambda: ops.varlen_prefill_attn(o, q, kf, vf, [L] * nseq,
+                                              D ** -0.5, tiles=ptiles), 5),
+        flops=4.0 * D * H * nseq * L * (L + 1) // 2)
+
+    # ---- decode attention: 64 sequences x 2048 cached, window 1024 ----
+    B, Lc = 64, 2048
+    nblk = B * (Lc // BS) + 1
+    bt = torch.arange(B * (Lc // BS), dtype=torch.int32, device=device).view(B, -1)
+    row_seq = torch.arange(B, dtype=torch.int32, device=device)
+    pos = torch.full((B,), Lc - 1, dtype=torch.int32, device=device)
+    kc = torch.randn(nblk, G, BS, D, device=device).to(bf)
+    vc = torch.randn(nblk, G, D, BS, device=device).to(bf)
+    qd = torch.randn(B, H, D, device=device).to(bf)
+    od = torch.empty_like(qd)
+    tiles = ops.build_attn_tiles(list(range(B)), [Lc - 1] * B, [1] * B, H, G, 1,
+                                 device)
+    rec("paged_attention decode, window 1024 + slopes (mfma)",
+        _time(lambda: ops.paged_attention(od, qd, kc, vc, bt, row_seq, pos,
+                                          D ** -0.5, window=win, tiles=tiles,
+                                          max_ctx=Lc, slopes=slopes)),
+        nbytes=B * win * G * D * 2 * 2)
+    kl = torch.randn(nblk, G, BS, D, device=device).to(bf)
+    vl = torch.randn_like(kl)
+    lens = torch.full((B,), Lc, dtype=torch.int32, device=device)
+    rec("paged_attn_decode (llama graph, 2048 keys)",
+        _time(lambda: ops.paged_attn_decode(od, qd, kl, vl, bt, lens, D ** -0.5)),
+        nbytes=B * Lc * G * D * 2 * 2)
+
+    # ---- row kernels at T = 8192 ----
+    T = 8192
+    x = torch.randn(T, W, device=device)
+    a = torch.randn(T, W, device=device).to(bf)
+    w32 = torch.ones(W, device=device)
+    hb = torch.empty(T, W, dtype=bf, device=device)
+    rec("add_layer_norm (add + layer norm, fp32 stream)",
+        _time(lambda: ops.add_layer_norm(x, a, w32, w32, 1e-5, hb)),
+        nbytes=T * W * 12)
+    xb, rb = a.clone(), a.clone()
+    wb = torch.ones(W, dtype=bf, device=device)
+    rec("fused_add_rms_norm (llama graph)",
+        _time(lambda: ops.fused_add_rms_norm(xb, rb, wb, 1e-6)),
+        nbytes=T * W * 8)
+    nblk = T // BS + 1
+    nq, nk = H * D, G * D
+    kc = torch.zeros(nblk, G, BS, D, dtype=bf, device=device)
+    vc = torch.zeros(nblk, G, D, BS, dtype=bf, device=device)
+    qkv = torch.randn(T, nq + 2 * nk, device=device).to(bf)
+    vfirst = torch.randn(T, nq + 2 * nk, device=device).to(bf)[:, nq + nk:]
+    qo = torch.empty(T, nq, dtype=bf, device=device)
+    wd = torch.ones(D, device=device)
+    lam = torch.tensor([0.3], device=device)
+    slots = torch.arange(T, device=device)
+    p32 = torch.arange(T, dtype=torch.int32, device=device)
+    pg = ops.build_page_groups([0], [0], [T], BS, device)
+    nb_store = T * (2 * nq + 2 * nk + 4 * nk) * 2   # q in/out, k in/out, v in, blend, back, page
+    rec("head_norm_store (head norms + temperature + blend + cache write, values by page)",
+        _time(lambda: ops.head_norm_store(qo, qkv, nq, nk, wd, wd, D, 0.1, 1024,
+                                          p32, vfirst, lam, kc, vc, slots, 1e-5,
+                                          page_groups=pg)),
+        nbytes=nb_store)
+    rec("head_norm_store, values row by row (decode's way)",
+        _time(lambda: ops.head_norm_store(qo, qkv, nq, nk, wd, wd, D, 0.1, 1024,
+                                          p32, vfirst, lam, kc, vc, slots, 1e-5)),
+        nbytes=T * (2 * nq + 2 * nk + 3 * nk) * 2)
+    qh = torch.randn(T, H, D, device=device).to(bf)
+    kk = torch.randn(T, G, D, device=device).to(bf)
+    kl = torch.zeros(nblk, G, BS, D, dtype=bf, device=device)
+    vl = torch.zeros_like(kl)
+    wn = torch.ones(D, dtype=bf, device=device)
+    cs = ops.build_cos_sin_cache(D, 64, T, 10000.0, None, device)
+    p64 = torch.arange(T, device=device)
+
+    def llama_chain():
+        ops.rms_norm(qh.view(-1, D), qh.view(-1, D), wn, 1e-6)
+        ops.rms_norm(kk.view(-1, D), kk.view(-1, D), wn, 1e-6)
+        ops.rotary_embedding(p64, qh, kk, cs, D, 64)
+        ops.reshape_and_cache(kk, kk, kl, vl, slots)
+
+    rec("rms_norm q, k + rotary_embedding + reshape_and_cache (llama graph)",
+        _time(llama_chain), nbytes=T * (2 * nq + 2 * nk + 3 * nk) * 2)
+    gu = torch.randn(T, 2 * s["ff"], device=device).to(bf)
+    ao = torch.empty(T, s["ff"], dtype=bf, device=device)
+    rec("act_and_mul silu", _time(lambda: ops.act_and_mul(ao, gu, "silu")),
+        nbytes=T * s["ff"] * 6)
+    rec("silu_and_mul (llama graph)", _time(lambda: ops.silu_and_mul(ao, gu)),
+        nbytes=T * s["ff"] * 6)
+
+    # ---- recurrent mixers ----
+    Hm, N, P, Gm, taps = 2 * W // 64, 128, 64, 8, 4
+    inner, gn = Hm * P, Gm * N
+    C = inner + 2 * gn
+    for label, nseq, L in (("prefill 8 x 1024", 8, 1024), ("decode 64 x 1", 64, 1)):
+        T = nseq * L
+        sf, sr = i32([i * L for i in range(nseq)]), i32([L] * nseq)
+        ss = i32(list(range(nseq)))
+        rs = torch.arange(nseq, dtype=torch.int32, device=device).repeat_interleave(L)
+        ps = (torch.arange(L, dtype=torch.int32, device=device) + 5).repeat(nseq)
+        u = torch.randn(T, 2 * inner + 2 * gn + Hm, device=device).to(bf)
+        xbc = torch.empty(T, C, dtype=bf, device=device)
+        cw, cb = torch.randn(C, taps, device=device), torch.zeros(C, device=device)
+        cst = torch.zeros(nseq + 1, taps - 1, C, dtype=bf, device=device)
+        rec(f"causal_conv_silu {label}",
+            _time(lambda: ops.causal_conv_silu(xbc, u, inner, cw, cb, cst, sf, sr,
+                                               ss, rs, ps)),
+            nbytes=T * C * 4)
+        y = torch.empty(T, inner, device=device)
+        st = torch.zeros(nseq + 1, Hm, N, P, device=device)
+        hv = torch.zeros(Hm, device=device)
+        sec = _time(lambda: ops.state_scan(y, xbc, 0, inner, inner + gn, u,
+                                           2 * inner + 2 * gn, Hm, Gm, N, P,
+                                           False, hv - 1, hv, hv + 1, None, st,
+                                           sf, sr, ss, ps), 5)
+        if L > 1:
+            rec(f"state_scan mamba2 {label} (fp32 vector ALU)", sec,
+                flops=4.0 * T * Hm * N * P, peak=PEAK_VALU)
+        else:
+            rec(f"state_scan mamba2 {label} (state read + write)", sec,
+                nbytes=nseq * Hm * N * P * 8)
+        # lightning: H heads of 128 x 128
+        ul = torch.randn(T, 4 * H * 128, device=device).to(bf)
+        yl = torch.empty(T, H * 128, device=device)
+        stl = torch.zeros(nseq + 1, H, 128, 128, device=device)
+        dec = torch.full((H,), 0.99, device=device)
+        sec = _time(lambda: ops.state_scan(yl, ul, 2 * H * 128, H * 128, 0, None,
+                                           0, H, H, 128, 128, True, None, None,
+                                           None, dec, stl, sf, sr, ss, ps), 5)
+        if L > 1:
+            rec(f"state_scan lightning {label} (fp32 vector ALU)", sec,
+                flops=4.0 * T * H * 128 * 128, peak=PEAK_VALU)
+        else:
+            rec(f"state_scan lightning {label} (state read + write)", sec,
+                nbytes=nseq * H * 128 * 128 * 8)
+        g = torch.empty(T, inner, dtype=bf, device=device)
+        wi = torch.ones(inner, device=device)
+        rec(f"gated_group_norm {label}",
+            _time(lambda: ops.gated_group_norm(g, y, u[:, :inner], wi, 8, 1e-5,
+                                               True)),
+            nbytes=T * inner * 8)
+    # ---- routing at T = 8192 ----
+    T, E = 8192, s["experts"]
+    lg = torch.randn(T, E, device=device)
+    ex = torch.empty(T, 4, dtype=torch.int32, device=device)
+    wt = torch.empty(T, 4, device=device)
+    corr = torch.zeros(E, device=device)
+    rec("route_topk (sigmoid + correction + top-2 group rank)",
+        _time(lambda: ops.route_topk(ex, wt, lg, corr, E, 4, 2, 2, True, True,
+                                     2.0)), nbytes=T * (E * 4 + 32))
+    rec("route_grouped_topk (softmax, best member)",
+        _time(lambda: ops.route_grouped_topk(ex, wt, lg, E, 4, 2, 2.0)),
+        nbytes=T * (E * 4 + 32))
+    return out
+
+
 def run(sizes: list[str], device: str, family: str = "vunitar") -> None:
     for name in sizes:
         s = SIZES[name]
-        for moe in ((False, True) if family == "vunitar" else (False,)):
+        if family == "livasun":
+            s = dict(s, layers=4)       # one full cycle of the three mixers
+        for moe in ((False, True) if family in ("vunitar", "livasun")
+                    else (False,)):
             row = {"size": name, **s, "ff_kind": "moe" if moe else "dense"}
-            mine = vunitar_spec if family == "vunitar" else fusipel_spec
+            mine = {"vunitar": vunitar_spec, "fusipel": fusipel_spec,
+                    "livasun": livasun_spec}[family]
             for label, mk in ((family, mine), ("llama_graph", llama_spec)):
                 pre, dec = engine_rates(mk(s, moe), device)
                 row[label] = {"prefill_tok_s": round(pre), "decode_tok_s": round(dec)}
             print(json.dumps({"layer_bench": row}), flush=True)
         if torch.cuda.is_available():
-            rates = kernel_rates if family == "vunitar" else fusipel_kernel_rates
+            rates = {"vunitar": kernel_rates, "fusipel": fusipel_kernel_rates,
+                     "livasun": livasun_kernel_rates}[family]
             for k in rates(s, device):
                 print(json.dumps({"kernel_bench": {"size": name, **k}}), flush=True)

@@ -78,6 +78,59 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
   st(out + (long)t * C + c, silu_f(acc));
 }
 
+// The same for bf16 rows whose channel count, first column and row stride
+// are multiples of 8: a lane takes 8 neighbouring channels of RB rows in a
+// row with 16-byte loads, its TAPS x 8 weights in registers.
+// grid (ceil(T / RB), ceil(C / 8 / 256)).
+constexpr int RB = 8;
+
+template <int TAPS>
+__global__ __launch_bounds__(256) void causal_conv_silu_vec_kernel(
+    unsigned short* __restrict__ out, const unsigned short* __restrict__ src,
+    long ld_src, int col0, int C, const float* __restrict__ w,
+    const float* __restrict__ b, const unsigned short* __restrict__ conv_state,
+    const int* __restrict__ seq_first, const int* __restrict__ state_slots,
+    const int* __restrict__ row_seq, const int* __restrict__ pos32, int nseq,
+    int nslots, int T) {
+  const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
+  if (c >= C) return;
+  constexpr int keep = TAPS - 1;
+  float wr[TAPS][8], br[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    br[e] = b[c + e];
+#pragma unroll
+    for (int k = 0; k < TAPS; ++k) wr[k][e] = w[(long)(c + e) * TAPS + k];
+  }
+  const int t_end = min(T, (int)(blockIdx.x + 1) * RB);
+  for (int t = blockIdx.x * RB; t < t_end; ++t) {
+    const int s = min(max(row_seq[t], 0), nseq - 1);
+    const int first = min(max(seq_first[s], 0), t);
+    const int i = t - first;
+    const int pos = max(pos32[t], 0);
+    const int slot = min(max(state_slots[s], 0), nslots - 1);
+    const unsigned short* stp = conv_state + (long)slot * keep * C;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = br[e];
+#pragma unroll
+    for (int k = 0; k < TAPS; ++k) {
+      const int d = keep - k;
+      u16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (i - d >= 0)
+        v = *reinterpret_cast<const u16x8*>(src + (long)(t - d) * ld_src + col0 + c);
+      else if (pos - d >= 0)
+        v = *reinterpret_cast<const u16x8*>(stp + (long)(keep + i - d) * C + c);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += wr[k][e] * bf2f(v[e]);
+    }
+    u16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = f2bf(silu_f(acc[e]));
+    *reinterpret_cast<u16x8*>(out + (long)t * C + c) = o;
+  }
+}
+
 // grid (nseq, ceil(C / 256)): the slot's new last inputs, after every read
 // of the old ones (stream order).
 template <typename TS>
@@ -221,6 +274,169 @@ __global__ __launch_bounds__(64) void state_scan_kernel(
   }
 }
 
+
+// The same recurrence for bf16 sources whose sizes and columns are multiples
+// of 8: four waves share one (sequence, head) and 4 * PL value channels, so
+// k and q are staged once for all of them with 16-byte loads; the next
+// CH rows are fetched into registers while the current ones are walked
+// (two LDS buffers, one barrier per pass). A lane owns the state rows
+// ns * NR .. ns * NR + NR - 1 and reads its k / q slice from LDS in 16-byte
+// pieces; slices of different ns sit NR + 4 floats apart, on other banks.
+template <int NR, int TPP>
+__global__ __launch_bounds__(256) void state_scan_vec_kernel(
+    float* __restrict__ y, const unsigned short* __restrict__ src,
+    const unsigned short* __restrict__ dt_src, ScanArgs p) {
+  constexpr int PL = 64 / TPP;
+  constexpr int NP = NR * TPP;
+  constexpr int NS = NR + 4;                 // floats between two ns slices
+  constexpr int ROW = TPP * NS;              // floats per staged k / q row
+  constexpr int PB = 4 * PL;                 // value channels per workgroup
+  constexpr int KV = (CH * NP / 8 + 255) / 256;   // 16-byte loads per lane
+  constexpr int VV = (CH * PB / 8 + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float ks[2][CH][ROW];
+  __shared__ __attribute__((aligned(16))) float qs[2][CH][ROW];
+  __shared__ float vs[2][CH][PB];
+  __shared__ float a_s[2][CH], b_s[2][CH];
+  const int s = blockIdx.x, h = blockIdx.y, pb0 = blockIdx.z * PB;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int pl = lane % PL, ns = lane / PL;
+  const int first = p.seq_first[s], n = p.seq_rows[s];
+  if (first < 0 || n < 1 || first + n > p.T) return;
+  const int slot = min(max(p.state_slots[s], 0), p.nslots - 1);
+  const int hist = p.pos32[first];
+  const int N = p.N, P = p.P;
+  const int g = h / (p.H / p.G);
+  const int pc = pb0 + wave * PL + pl;
+  const bool live = pc < P;
+  float* sp = p.state + ((long)slot * p.H + h) * N * P;
+  float S[NR];
+#pragma unroll
+  for (int j = 0; j < NR; ++j) {
+    const int nn = ns * NR + j;
+    S[j] = (hist > 0 && live && nn < N) ? sp[(long)nn * P + pc] : 0.f;
+  }
+  const float skip = p.skip != nullptr ? p.skip[h] : 0.f;
+  const float a_rate = dt_src != nullptr ? expf(p.a_log[h]) : 0.f;
+  const float dtb = dt_src != nullptr ? p.dt_bias[h] : 0.f;
+  const float a_const = dt_src == nullptr ? p.decay[h] : 0.f;
+  const int nvec = N / 8;                    // 16-byte pieces per k / q row
+  const u16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  u16x8 kreg[KV], qreg[KV], vreg[VV];
+  float dreg = 0.f;
+  auto fetch = [&](int c0) {
+    const int rows = min(CH, n - c0);
+#pragma unroll
+    for (int u = 0; u < KV; ++u) {
+      const int i = tid + u * 256;
+      kreg[u] = zero8;
+      qreg[u] = zero8;
+      if (i < rows * nvec) {
+        const int r = i / nvec, e = (i % nvec) * 8;
+        const unsigned short* rp = src + (long)(first + c0 + r) * p.ld_src;
+        kreg[u] = *reinterpret_cast<const u16x8*>(rp + p.col_b + g * N + e);
+        qreg[u] = *reinterpret_cast<const u16x8*>(rp + p.col_c + g * N + e);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < VV; ++u) {
+      const int i = tid + u * 256;
+      vreg[u] = zero8;
+      if (i < rows * (PB / 8)) {
+        const int r = i / (PB / 8), c = (i % (PB / 8)) * 8;
+        if (pb0 + c < P)
+          vreg[u] = *reinterpret_cast<const u16x8*>(
+              src + (long)(first + c0 + r) * p.ld_src + p.col_x + h * P + pb0 + c);
+      }
+    }
+    if (dt_src != nullptr && tid < rows)
+      dreg = bf2f(dt_src[(long)(first + c0 + tid) * p.ld_dt + p.col_dt + h]);
+  };
+  auto stage = [&](int buf, int c0) {
+    const int rows = min(CH, n - c0);
+#pragma unroll
+    for (int u = 0; u < KV; ++u) {
+      const int i = tid + u * 256;
+      if (i < rows * nvec) {
+        const int r = i / nvec, e = (i % nvec) * 8;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          float kv = bf2f(kreg[u][k]), qv = bf2f(qreg[u][k]);
+          if (p.act) { kv = silu_f(kv); qv = silu_f(qv); }
+          const int nn = e + k;
+          const int at = (nn / NR) * NS + nn % NR;
+          ks[buf][r][at] = kv;
+          qs[buf][r][at] = qv;
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < VV; ++u) {
+      const int i = tid + u * 256;
+      if (i < rows * (PB / 8)) {
+        const int r = i / (PB / 8), c = (i % (PB / 8)) * 8;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          float v = bf2f(vreg[u][k]);
+          if (p.act) v = silu_f(v);
+          vs[buf][r][c + k] = v;
+        }
+      }
+    }
+    if (tid < rows) {
+      if (dt_src != nullptr) {
+        const float dt = softplus_f(dreg + dtb);
+        a_s[buf][tid] = expf(-a_rate * dt);
+        b_s[buf][tid] = dt;
+      } else {
+        a_s[buf][tid] = a_const;
+        b_s[buf][tid] = 1.f;
+      }
+    }
+  };
+  // state rows past N (padding up to NP) keep k = q = 0: zero them once
+  for (int i = tid; i < 2 * CH * ROW; i += 256) {
+    (&ks[0][0][0])[i] = 0.f;
+    (&qs[0][0][0])[i] = 0.f;
+  }
+  __syncthreads();
+  fetch(0);
+  int buf = 0;
+  for (int c0 = 0; c0 < n; c0 += CH, buf ^= 1) {
+    const int rows = min(CH, n - c0);
+    stage(buf, c0);
+    __syncthreads();
+    if (c0 + CH < n) fetch(c0 + CH);
+    const float* kb = &ks[buf][0][ns * NS];
+    const float* qb = &qs[buf][0][ns * NS];
+    for (int r = 0; r < rows; ++r) {
+      const float a = a_s[buf][r];
+      const float v = vs[buf][r][wave * PL + pl];
+      const float bv = b_s[buf][r] * v;
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < NR; j += 4) {
+        const f32x4 k4 = *reinterpret_cast<const f32x4*>(kb + r * ROW + j);
+        const f32x4 q4 = *reinterpret_cast<const f32x4*>(qb + r * ROW + j);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          S[j + k] = a * S[j + k] + k4[k] * bv;
+          acc += S[j + k] * q4[k];
+        }
+      }
+#pragma unroll
+      for (int m = PL; m < 64; m <<= 1) acc += __shfl_xor(acc, m, WAVE_SIZE);
+      if (ns == 0 && live)
+        y[(long)(first + c0 + r) * p.H * P + h * P + pc] = acc + skip * v;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < NR; ++j) {
+    const int nn = ns * NR + j;
+    if (live && nn < N) sp[(long)nn * P + pc] = S[j];
+  }
+}
+
 constexpr int ROW_THREADS = 256;
 
 DEVICE_INLINE float block_sum(float v, float* red) {
@@ -279,9 +495,28 @@ bool scan_pick(float* y, const void* src, const void* dt, const ScanArgs& p,
   int tpp = 1;
   while (tpp < 8 && ((p.N + tpp - 1) / tpp > 32 || 64 / tpp > max(p.P, 8)))
     tpp *= 2;
+  // 16-byte staging: bf16 rows whose sizes and columns are multiples of 8
+  const bool vec = p.N % 8 == 0 && p.P % 8 == 0 &&
+                   p.ld_src % 8 == 0 && p.col_x % 8 == 0 && p.col_b % 8 == 0 &&
+                   p.col_c % 8 == 0;
+  // few workgroups (long portions of few sequences): more lanes per channel
+  // make more, smaller ones, so that every SIMD holds two waves
+  while (vec && sizeof(TS) == 2 && tpp < 8 && (p.N + tpp - 1) / tpp >= 16 &&
+         (long)nseq * p.H * ((p.P + 4 * (64 / tpp) - 1) / (4 * (64 / tpp))) < 512)
+    tpp *= 2;
   const int nr = (p.N + tpp - 1) / tpp;
 #define SCAN_CASE(NRV, TPPV)                                              \
   if (tpp == TPPV && nr <= NRV) {                                         \
+    constexpr bool fits = sizeof(TS) == 2 &&                              \
+        (4 * CH * TPPV * (NRV + 4) + 2 * CH * 4 * (64 / TPPV) + 4 * CH) * 4 \
+            <= 60 * 1024;                                                 \
+    if constexpr (fits) if (vec) {                                        \
+      constexpr int PBV = 4 * (64 / TPPV);                                \
+      dim3 grid(nseq, p.H, (p.P + PBV - 1) / PBV);                        \
+      state_scan_vec_kernel<NRV, TPPV><<<grid, 256, 0, s>>>(              \
+          y, (const unsigned short*)src, (const unsigned short*)dt, p);   \
+      return true;                                                        \
+    }                                                                     \
     scan_launch<TS, TD, NRV, TPPV>(y, src, dt, p, nseq, s);               \
     return true;                                                          \
   }
@@ -307,10 +542,24 @@ void causal_conv_silu_launch(void* out, const void* src, long ld_src, int col0,
   if (T <= 0 || nseq <= 0) return;
   dim3 grid(T, (C + 255) / 256), sgrid(nseq, (C + 255) / 256);
   if (bf) {
-    causal_conv_silu_kernel<unsigned short><<<grid, 256, 0, s>>>(
-        (unsigned short*)out, (const unsigned short*)src, ld_src, col0, C, taps,
-        w, b, (const unsigned short*)conv_state, seq_first, state_slots,
-        row_seq, pos32, nseq, nslots, T);
+    // few rows (decode): one lane per (row, channel) makes more workgroups
+    const bool vec = C % 8 == 0 && col0 % 8 == 0 && ld_src % 8 == 0 &&
+                     (long)T * C >= (1 << 20);
+    const dim3 vgrid((T + RB - 1) / RB, (C / 8 + 255) / 256);
+#define CONV_VEC(TAPSV)                                                        \
+  causal_conv_silu_vec_kernel<TAPSV><<<vgrid, 256, 0, s>>>(                    \
+      (unsigned short*)out, (const unsigned short*)src, ld_src, col0, C, w, b, \
+      (const unsigned short*)conv_state, seq_first, state_slots, row_seq,      \
+      pos32, nseq, nslots, T)
+    if (vec && taps == 4) CONV_VEC(4);
+    else if (vec && taps == 3) CONV_VEC(3);
+    else if (vec && taps == 2) CONV_VEC(2);
+#undef CONV_VEC
+    else
+      causal_conv_silu_kernel<unsigned short><<<grid, 256, 0, s>>>(
+          (unsigned short*)out, (const unsigned short*)src, ld_src, col0, C,
+          taps, w, b, (const unsigned short*)conv_state, seq_first, state_slots,
+          row_seq, pos32, nseq, nslots, T);
     if (taps > 1)
       conv_state_update_kernel<unsigned short><<<sgrid, 256, 0, s>>>(
           (const unsigned short*)src, ld_src, col0, C, taps,

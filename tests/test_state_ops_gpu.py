@@ -133,10 +133,15 @@ def test_route_topk(sigmoid, E, G, keep, gtop, top):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("taps", [1, 2, 4, 7])
-def test_causal_conv_silu(dtype, taps):
-    C, col0, ld = 300, 17, 400
-    news, hists, slots = [9, 1, 1, 2, 30, 1], [0, 5, 0, 1, 2, 1], [3, 0, 5, 1, 2, 4]
+@pytest.mark.parametrize("taps", [1, 2, 3, 4, 7])
+@pytest.mark.parametrize("C,col0,big", [(300, 17, 1), (304, 16, 1),
+                                        (2056, 8, 1), (2056, 8, 500)])
+def test_causal_conv_silu(dtype, taps, C, col0, big):
+    """(2056, 8) with the long portion: the 16-byte row-blocked kernel in
+    bf16 (2, 3 or 4 taps); the others one lane per (row, channel)."""
+    ld = C + col0 + 16
+    news, hists, slots = ([9, 1, 1, 2, 30 * big, 1], [0, 5, 0, 1, 2, 1],
+                          [3, 0, 5, 1, 2, 4])
     view = _ragged(news, hists, slots)
     T = sum(news)
     src = _rand(T, ld, dtype=dtype)
@@ -162,14 +167,18 @@ def test_causal_conv_silu(dtype, taps):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("H,G,N,P", [
     (4, 2, 32, 32), (4, 4, 64, 32), (3, 1, 24, 20), (2, 2, 128, 64),
-    (2, 1, 200, 8), (5, 5, 16, 100), (2, 2, 256, 16), (6, 3, 7, 3)])
+    (2, 1, 200, 8), (5, 5, 16, 100), (2, 2, 256, 16), (6, 3, 7, 3),
+    (2, 1, 64, 128), (3, 3, 24, 40), (2, 2, 8, 8), (2, 1, 128, 24)])
 @pytest.mark.parametrize("stepped", [True, False])
-def test_state_scan(dtype, H, G, N, P, stepped):
+@pytest.mark.parametrize("off", [3, 8])
+def test_state_scan(dtype, H, G, N, P, stepped, off):
+    """off = 8 with sizes that are multiples of 8 takes the 16-byte staging
+    kernel in bf16; everything else the plain one."""
     news, hists, slots = [21, 1, 1, 2, 40], [0, 5, 0, 1, 2], [3, 0, 5, 1, 2]
     sf, sr, ss, _, pos = _ragged(news, hists, slots)
     T = sum(news)
-    cx, cb, cc, cdt = 3, 3 + H * P, 3 + H * P + G * N, 3 + H * P + 2 * G * N
-    src = _rand(T, cdt + H + 2, dtype=dtype, std=0.7)
+    cx, cb, cc, cdt = off, off + H * P, off + H * P + G * N, off + H * P + 2 * G * N
+    src = _rand(T, (cdt + H + 9) // 8 * 8, dtype=dtype, std=0.7)
     st0 = _rand(7, H, N, P, seed=5)
     if stepped:
         extra = (src, cdt, H, G, N, P, False, _rand(H, seed=6) - 1,
