@@ -158,8 +158,11 @@ def test_causal_conv_silu(dtype, taps, C, col0, big):
             torch_ref.causal_conv_silu(out, src, col0, w, b, st, view[0],
                                        view[1], view[2], view[4])
         res.append((out, st))
-    tol = 0.03 if dtype == torch.bfloat16 else 1e-5
-    assert (res[0][0].float() - res[1][0].float()).abs().max() <= tol
+    got, ref = res[0][0].float(), res[1][0].float()
+    if dtype == torch.bfloat16:     # one bf16 step of the value at most
+        assert ((got - ref).abs() <= 0.008 * ref.abs() + 0.004).all()
+    else:
+        assert (got - ref).abs().max() <= 1e-5
     assert torch.equal(res[0][1], res[1][1])        # inputs are copied as is
     assert torch.equal(res[0][1][6], st0[6])        # an unused slot is untouched
 
