@@ -477,6 +477,54 @@ __global__ __launch_bounds__(ROW_THREADS) void gated_group_norm_kernel(
   }
 }
 
+// The same for bf16 gates and outputs with parts of a multiple of 4 and at
+// most 4096 channels: a lane keeps its 4 x NV channels in registers between
+// the sum of squares and the store (one pass over y and the gate).
+template <int NV>
+__global__ __launch_bounds__(ROW_THREADS) void gated_group_norm_vec_kernel(
+    unsigned short* __restrict__ out, const float* __restrict__ y,
+    const unsigned short* __restrict__ gate, long ld_gate,
+    const float* __restrict__ w, int C, int gs, float eps, int gate_first) {
+  __shared__ float red[4];
+  const long t = blockIdx.x;
+  const int c0 = blockIdx.y * gs;
+  const float* yr = y + t * C + c0;
+  const unsigned short* gr = gate + t * ld_gate + c0;
+  float u[NV][4], gv[NV][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int i = (threadIdx.x + j * ROW_THREADS) * 4;
+    if (i < gs) {
+      const f32x4 yv = *reinterpret_cast<const f32x4*>(yr + i);
+      const u16x4 g4 = *reinterpret_cast<const u16x4*>(gr + i);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        gv[j][k] = bf2f(g4[k]);
+        u[j][k] = gate_first ? yv[k] * silu_f(gv[j][k]) : yv[k];
+        ss += u[j][k] * u[j][k];
+      }
+    }
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)gs + eps);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int i = (threadIdx.x + j * ROW_THREADS) * 4;
+    if (i < gs) {
+      const f32x4 wv = *reinterpret_cast<const f32x4*>(w + c0 + i);
+      u16x4 o;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float r = u[j][k] * inv * wv[k];
+        if (!gate_first) r *= sigmoid_f(gv[j][k]);
+        o[k] = f2bf(r);
+      }
+      *reinterpret_cast<u16x4*>(out + t * C + c0 + i) = o;
+    }
+  }
+}
+
 template <typename TS, typename TD, int NR, int TPP>
 void scan_launch(float* y, const void* src, const void* dt, const ScanArgs& p,
                  int nseq, hipStream_t s) {
@@ -607,6 +655,18 @@ void gated_group_norm_launch(void* out, const float* y, const void* gate,
   if (T <= 0) return;
   dim3 grid(T, groups);
   const int gs = C / groups;
+  if (gate_bf && out_bf && gs % 4 == 0 && C % 4 == 0 && ld_gate % 4 == 0 &&
+      gs <= 4096 && ((uintptr_t)gate % 8) == 0) {
+    if (gs <= 1024)
+      gated_group_norm_vec_kernel<1><<<grid, ROW_THREADS, 0, s>>>(
+          (unsigned short*)out, y, (const unsigned short*)gate, ld_gate, w, C,
+          gs, eps, gate_first);
+    else
+      gated_group_norm_vec_kernel<4><<<grid, ROW_THREADS, 0, s>>>(
+          (unsigned short*)out, y, (const unsigned short*)gate, ld_gate, w, C,
+          gs, eps, gate_first);
+    return;
+  }
   if (gate_bf) {
     if (out_bf)
       gated_group_norm_kernel<unsigned short, unsigned short>

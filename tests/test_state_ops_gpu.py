@@ -203,12 +203,17 @@ def test_state_scan(dtype, H, G, N, P, stepped, off):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("C,groups", [(128, 2), (96, 1), (300, 3), (2048, 8)])
-def test_gated_group_norm(out_dtype, C, groups):
+@pytest.mark.parametrize("C,groups,col", [(128, 2, 4), (96, 1, 4), (300, 3, 4),
+                                          (2048, 8, 4), (2048, 8, 8),
+                                          (6000, 2, 16), (1000, 5, 0),
+                                          (20000, 4, 8)])
+def test_gated_group_norm(out_dtype, C, groups, col):
+    """Gate columns at multiples of 4 elements take the one-pass kernel in
+    bf16 (parts up to 4096 channels)."""
     T = 11
     y = _rand(T, C, std=3.0)
-    gsrc = _rand(T, C + 10, dtype=out_dtype, seed=2)
-    gate = gsrc[:, 4:4 + C]
+    gsrc = _rand(T, C + 24, dtype=out_dtype, seed=2)
+    gate = gsrc[:, col:col + C]
     w = _rand(C, seed=3)
     for first in (True, False):
         o = torch.zeros(T, C, dtype=out_dtype, device=DEV)
