@@ -611,13 +611,13 @@ class ModelSpec:
                     qk_dim=int(m["dim"]), v_dim=int(m.get("vdim", m["dim"])),
                     scale=float(m["scale"]),
                     window=int(mask.get("size", 0) or 0), head_norm=True,
-                    q_temp=(float(qt["coef"]), int(qt["every"]))
+                    q_temp=(float(qt["coef"]), float(qt["every"]))
                     if qt else None,
                     distance_bias=True, v_mix=bool(m.get("v_mix", False)))
                 if mixer.heads % mixer.kv_heads:
                     raise ValueError("heads must be a multiple of kv_heads")
-                if mixer.q_temp is not None and mixer.q_temp[1] < 1:
-                    raise ValueError("q_temp.every must be at least 1")
+                if mixer.q_temp is not None and not mixer.q_temp[1] > 0:
+                    raise ValueError("q_temp.every must be positive")
                 mtype = "paged_attention"
             elif kind == "mamba2":
                 mixer = ScanMixerSpec(

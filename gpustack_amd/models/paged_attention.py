@@ -113,7 +113,7 @@ class PagedRotaryAttention(nn.Module):
             v_first = None
             if m.v_mix and not self.v_mix_first:
                 v_first = shared["v_first"]
-            coef, every = m.q_temp or (0.0, 0)
+            coef, every = m.q_temp or (0.0, 0.0)
             ops.head_norm_store(q, qkv, self.nq, self.nk, self.q_head_norm,
                                 self.k_head_norm, m.qk_dim, coef, every,
                                 rg.pos32, v_first, self.v_lam, k_cache,

@@ -779,7 +779,7 @@ def add_layer_norm(x, a, w, b, eps: float, h) -> None:
 
 
 def head_norm_store(q_out, qkv, nq: int, nk: int, q_w, k_w, head_dim: int,
-                    temp_coef: float, temp_every: int, pos32, v_first, lam,
+                    temp_coef: float, temp_every: float, pos32, v_first, lam,
                     k_cache, v_cache, slots, eps: float,
                     page_groups=None) -> None:
     """`page_groups` (build_page_groups; GPU, prompts): the value rows are

@@ -118,7 +118,7 @@ template <typename TS, typename TC>
 __global__ __launch_bounds__(ROW_THREADS) void head_norm_store_kernel(
     TS* __restrict__ q_out, TS* __restrict__ qkv, long ld_qkv, int nq, int nk,
     int nv, const float* __restrict__ q_w, const float* __restrict__ k_w,
-    int D, float temp_coef, int temp_every, const int* __restrict__ pos32,
+    int D, float temp_coef, float temp_every, const int* __restrict__ pos32,
     const TS* __restrict__ v_first, long ld_vf, const float* __restrict__ lam,
     TC* __restrict__ k_cache, TC* __restrict__ v_cache,
     const long* __restrict__ slots, long nslots, int G, int BS, int VW,
@@ -131,9 +131,10 @@ __global__ __launch_bounds__(ROW_THREADS) void head_norm_store_kernel(
   const long blk = keep ? slot / BS : 0;
   const int off = keep ? (int)(slot % BS) : 0;
   float temp = 1.f;
-  if (temp_every > 0) {
+  if (temp_every > 0.f) {
+    // exact for whole-numbered steps while the position is below 2^24
     const int p = max(pos32[t], 0);
-    temp = 1.f + temp_coef * logf((float)((p + 1) / temp_every) + 1.f);
+    temp = 1.f + temp_coef * logf(floorf((float)(p + 1) / temp_every) + 1.f);
   }
   const int HQ = nq / D;
   for (int hd = wave; hd < HQ + G; hd += 4) {
@@ -334,7 +335,7 @@ void add_layer_norm_launch(float* x, const void* a, const float* w,
 
 void head_norm_store_launch(void* q_out, void* qkv, long ld_qkv, int nq, int nk,
                             int nv, const float* q_w, const float* k_w, int D,
-                            float temp_coef, int temp_every, const int* pos32,
+                            float temp_coef, float temp_every, const int* pos32,
                             const void* v_first, long ld_vf, const float* lam,
                             void* k_cache, void* v_cache, const long* slots,
                             long nslots, int G, int BS, int VW, float eps,

@@ -9,7 +9,7 @@
 
 void embed_rows_scaled_launch(float*, const long*, const void*, int, int, long, float, int, hipStream_t);
 void add_layer_norm_launch(float*, const void*, const float*, const float*, void*, int, int, float, int, int, hipStream_t);
-void head_norm_store_launch(void*, void*, long, int, int, int, const float*, const float*, int, float, int, const int*, const void*, long, const float*, void*, void*, const long*, long, int, int, int, float, int, int, int, hipStream_t);
+void head_norm_store_launch(void*, void*, long, int, int, int, const float*, const float*, int, float, float, const int*, const void*, long, const float*, void*, void*, const long*, long, int, int, int, float, int, int, int, hipStream_t);
 void value_page_store_launch(const void*, long, int, void*, const long*, long, const int*, int, int, int, int, int, hipStream_t);
 void route_topk_launch(int*, float*, const float*, int, const float*, int, int, int, int, int, int, int, int, float, hipStream_t);
 void causal_conv_silu_launch(void*, const void*, long, int, int, int, const float*, const float*, void*, const int*, const int*, const int*, const int*, const int*, int, int, int, int, hipStream_t);
@@ -103,7 +103,7 @@ void add_layer_norm(Tensor x, OptTensor a, OptTensor w, OptTensor b, double eps,
 
 void head_norm_store(Tensor q_out, Tensor qkv, long nq, long nk, Tensor q_w,
                      Tensor k_w, long head_dim, double temp_coef,
-                     long temp_every, Tensor pos32, OptTensor v_first,
+                     double temp_every, Tensor pos32, OptTensor v_first,
                      OptTensor lam, Tensor k_cache, Tensor v_cache, Tensor slots,
                      double eps, OptTensor page_groups) {
   const int bf = act_kind(q_out, "q_out");
@@ -145,7 +145,7 @@ void head_norm_store(Tensor q_out, Tensor qkv, long nq, long nk, Tensor q_w,
   head_norm_store_launch(q_out.data_ptr(), qkv.data_ptr(), qkv.stride(0),
                          (int)nq, (int)nk, (int)nv, q_w.data_ptr<float>(),
                          k_w.data_ptr<float>(), D, (float)temp_coef,
-                         (int)temp_every, pos32.data_ptr<int>(), vf, ld_vf, lp,
+                         (float)temp_every, pos32.data_ptr<int>(), vf, ld_vf, lp,
                          k_cache.data_ptr(), v_cache.data_ptr(),
                          slots.data_ptr<long>(), k_cache.size(0) * (long)BS, G,
                          BS, VW, (float)eps, page_groups.has_value() ? 1 : 0, T,

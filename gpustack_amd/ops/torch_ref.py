@@ -622,7 +622,7 @@ def add_layer_norm(x: torch.Tensor, a: torch.Tensor | None,
 
 def head_norm_store(q_out: torch.Tensor, qkv: torch.Tensor, nq: int, nk: int,
                     q_w: torch.Tensor, k_w: torch.Tensor, head_dim: int,
-                    temp_coef: float, temp_every: int, pos32: torch.Tensor,
+                    temp_coef: float, temp_every: float, pos32: torch.Tensor,
                     v_first: torch.Tensor | None, lam: torch.Tensor | None,
                     k_cache: torch.Tensor, v_cache: torch.Tensor,
                     slots: torch.Tensor, eps: float) -> None:

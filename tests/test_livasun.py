@@ -232,8 +232,10 @@ def test_feed_forwards_alone(tmp_path):
     [oracle.attn_layer(heads=3, kv_heads=3, dim=8, vdim=8),
      oracle.mamba_layer(heads=2, groups=2, state=9, vdim=3, conv=2,
                         norm_groups=1)],
-    # one kv head, one head, one group, one tap, window of one key
-    [oracle.attn_layer(heads=5, kv_heads=1, dim=6, vdim=4, window=1),
+    # one kv head, one head, one group, one tap, window of one key ...
+    # ... and a temperature step that is no whole number
+    [oracle.attn_layer(heads=5, kv_heads=1, dim=6, vdim=4, window=1,
+                       temp=(0.7, 2.5)),
      oracle.mamba_layer(heads=1, groups=1, state=4, vdim=8, conv=1,
                         norm_groups=4),
      oracle.lightning_layer(heads=1, dim=5, vdim=9, decay=(1.0,))],
