@@ -103,7 +103,7 @@ def livasun_spec(s, moe: bool = False):
     if moe:
         ff = FeedForwardSpec(kind="moe", ff=s["eff"], act="relu2",
                              experts=s["experts"], top=4, groups=4,
-                             keep_groups=2, route_scale=2.0,
+                             keep_groups=2, route_scale=2.5,
                              shared_ff=s["eff"], route_scores="sigmoid",
                              route_correction=True, group_top=2, renorm=True)
     else:

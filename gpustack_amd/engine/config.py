@@ -348,6 +348,15 @@ class ModelSpec:
                 out.append(None)
         return out
 
+    def state_bytes_per_slot(self, dtype_size: int = 2) -> int:
+        """Bytes one live sequence holds in the recurrent-state pool: fp32
+        matrix states plus the convolutions' last inputs in the engine
+        dtype, over all layer runs."""
+        if self.layers is None:
+            return 0
+        return sum(sh[0] * sh[1] * sh[2] * 4 + sh[3] * sh[4] * dtype_size
+                   for sh in self.state_pool_shapes() if sh is not None)
+
     @property
     def has_state(self) -> bool:
         return self.layers is not None and any(

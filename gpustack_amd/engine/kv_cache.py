@@ -374,6 +374,10 @@ class KVCache:
         esize = 1 if cfg.kv_cache_dtype == "fp8" else 2
         if spec.layers is not None:
             esize = 4 if cfg.dtype == "float32" else 2
+            # the state pool (one slot per admissible sequence and a spare)
+            # comes out of the same memory before the paged pools are sized
+            free_bytes = max(0, free_bytes - (cfg.max_num_seqs + 1)
+                             * spec.state_bytes_per_slot(esize))
             planes = KVCache.latent_planes(cfg)
             per_block = max(1, cfg.block_size * esize * sum(
                 w[1] * planes if w[0] == "latent" else

@@ -180,17 +180,18 @@ struct ScanArgs {
 constexpr int CH = 16;     // rows staged per pass
 
 // One wave per (sequence, head, block of PL = 64 / TPP value channels).
-// lane = ns * PL + pl: channel p0 + pl, state rows n = r * TPP + ns.
-template <typename TS, typename TD, int NR, int TPP>
+// lane = ns * PL + pl: channel p0 + pl, state rows n = r * TPP + ns. CHG rows
+// are staged per pass (fewer for the widest states, to fit the LDS).
+template <typename TS, typename TD, int NR, int TPP, int CHG>
 __global__ __launch_bounds__(64) void state_scan_kernel(
     float* __restrict__ y, const TS* __restrict__ src,
     const TD* __restrict__ dt_src, ScanArgs p) {
   constexpr int PL = 64 / TPP;
   constexpr int NP = NR * TPP;               // padded state rows
-  __shared__ float ks[CH][NP];
-  __shared__ float qs[CH][NP];
-  __shared__ float vs[CH][PL];
-  __shared__ float a_s[CH], b_s[CH];
+  __shared__ float ks[CHG][NP];
+  __shared__ float qs[CHG][NP];
+  __shared__ float vs[CHG][PL];
+  __shared__ float a_s[CHG], b_s[CHG];
   const int s = blockIdx.x, h = blockIdx.y, p0 = blockIdx.z * PL;
   const int lane = threadIdx.x;
   const int pl = lane % PL, ns = lane / PL;
@@ -214,8 +215,8 @@ __global__ __launch_bounds__(64) void state_scan_kernel(
   const float dtb = dt_src != nullptr ? p.dt_bias[h] : 0.f;
   const float a_const = dt_src == nullptr ? p.decay[h] : 0.f;
 
-  for (int c0 = 0; c0 < n; c0 += CH) {
-    const int rows = min(CH, n - c0);
+  for (int c0 = 0; c0 < n; c0 += CHG) {
+    const int rows = min(CHG, n - c0);
     __syncthreads();
     for (int i = lane; i < rows * NP; i += 64) {
       const int r = i / NP, nn = i % NP;
@@ -530,8 +531,8 @@ void scan_launch(float* y, const void* src, const void* dt, const ScanArgs& p,
                  int nseq, hipStream_t s) {
   constexpr int PL = 64 / TPP;
   dim3 grid(nseq, p.H, (p.P + PL - 1) / PL);
-  state_scan_kernel<TS, TD, NR, TPP><<<grid, 64, 0, s>>>(
-      y, (const TS*)src, (const TD*)dt, p);
+  state_scan_kernel<TS, TD, NR, TPP, (NR * TPP > 256 ? 8 : 16)>
+      <<<grid, 64, 0, s>>>(y, (const TS*)src, (const TD*)dt, p);
 }
 
 // Rows of the state per lane (NR) and lanes per value channel (TPP): the
@@ -570,7 +571,7 @@ bool scan_pick(float* y, const void* src, const void* dt, const ScanArgs& p,
   }
 #define SCAN_TPP(TPPV) \
   SCAN_CASE(4, TPPV) SCAN_CASE(8, TPPV) SCAN_CASE(16, TPPV) SCAN_CASE(32, TPPV)
-  SCAN_TPP(1) SCAN_TPP(2) SCAN_TPP(4) SCAN_TPP(8)
+  SCAN_TPP(1) SCAN_TPP(2) SCAN_TPP(4) SCAN_TPP(8) SCAN_CASE(64, 8)
 #undef SCAN_TPP
 #undef SCAN_CASE
   return false;
@@ -578,7 +579,7 @@ bool scan_pick(float* y, const void* src, const void* dt, const ScanArgs& p,
 
 }  // namespace
 
-int state_scan_max_state() { return 8 * 32; }
+int state_scan_max_state() { return 8 * 64; }
 int conv_max_taps() { return MAX_TAPS; }
 
 void causal_conv_silu_launch(void* out, const void* src, long ld_src, int col0,

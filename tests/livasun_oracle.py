@@ -276,7 +276,7 @@ def moe(experts=6, count=3, keep=2, top=2, ff=10, shared=12, scale=1.5):
     return f
 
 
-def make_config(width=24, vocab=53, layers=None, embed_scale=3.0, eps=1e-5):
+def make_config(width=24, vocab=53, layers=None, embed_scale=3.0, eps=1e-6):
     if layers is None:
         layers = [attn_layer(mlp=dense()),
                   mamba_layer(mlp=moe()),

@@ -24,10 +24,10 @@ pytestmark = pytest.mark.gpu
 # other
 ALIGNED = dict(width=64, vocab=97, layers=[
     oracle.attn_layer(heads=4, kv_heads=2, dim=32, vdim=16, window=37,
-                      temp=(0.3, 20), mlp=oracle.dense(80)),
+                      temp=(0.25, 20), mlp=oracle.dense(80)),
     oracle.mamba_layer(heads=4, groups=2, state=16, vdim=24, conv=4,
                        norm_groups=3,
-                       mlp=oracle.moe(experts=8, count=4, keep=3, top=3, ff=64,
+                       mlp=oracle.moe(experts=8, count=2, keep=1, top=3, ff=64,
                                       shared=40)),
     oracle.attn_layer(heads=6, kv_heads=2, dim=64, vdim=16, window=0,
                       temp=None),
