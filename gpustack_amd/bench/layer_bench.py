@@ -632,7 +632,7 @@ def livasun_kernel_rates(s, device):
         sec = _time(lambda: ops.state_scan(y, xbc, 0, inner, inner + gn, u,
                                            2 * inner + 2 * gn, Hm, Gm, N, P,
                                            False, hv - 1, hv, hv + 1, None, st,
-                                           sf, sr, ss, ps), 5)
+                                           sf, sr, ss, ps, single=L == 1), 5)
         if L > 1:
             rec(f"state_scan mamba2 {label} (fp32 vector ALU)", sec,
                 flops=4.0 * T * Hm * N * P, peak=PEAK_VALU)
@@ -646,7 +646,8 @@ def livasun_kernel_rates(s, device):
         dec = torch.full((H,), 0.99, device=device)
         sec = _time(lambda: ops.state_scan(yl, ul, 2 * H * 128, H * 128, 0, None,
                                            0, H, H, 128, 128, True, None, None,
-                                           None, dec, stl, sf, sr, ss, ps), 5)
+                                           None, dec, stl, sf, sr, ss, ps,
+                                           single=L == 1), 5)
         if L > 1:
             rec(f"state_scan lightning {label} (fp32 vector ALU)", sec,
                 flops=4.0 * T * H * 128 * 128, peak=PEAK_VALU)

@@ -72,7 +72,8 @@ class Mamba2Mixer(nn.Module):
         ops.state_scan(y, xbc, 0, m.inner, m.inner + gn, u, self.col_dt,
                        m.heads, m.groups, m.state, m.vdim, False,
                        self.dt_bias, self.a_log, self.skip, None, ssm_state,
-                       rg.seq_first, rg.seq_rows, rg.state_slots, rg.pos32)
+                       rg.seq_first, rg.seq_rows, rg.state_slots, rg.pos32,
+                       single=max(rg.seq_news, default=1) <= 1)
         g = torch.empty(T, m.inner, dtype=h.dtype, device=h.device)
         ops.gated_group_norm(g, y, u[:, :m.inner], self.norm, m.norm_groups,
                              self.eps, True)
@@ -107,7 +108,8 @@ class LightningMixer(nn.Module):
         ops.state_scan(y, u, 2 * self.nqk, self.nqk, 0, None, 0, m.heads,
                        m.heads, m.state, m.vdim, True, None, None, None,
                        self.decay, ssm_state, rg.seq_first, rg.seq_rows,
-                       rg.state_slots, rg.pos32)
+                       rg.state_slots, rg.pos32,
+                       single=max(rg.seq_news, default=1) <= 1)
         g = torch.empty(T, m.inner, dtype=h.dtype, device=h.device)
         ops.gated_group_norm(g, y, u[:, 2 * self.nqk + m.inner:], self.norm,
                              1, self.eps, False)

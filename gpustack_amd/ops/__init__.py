@@ -809,12 +809,15 @@ def causal_conv_silu(out, src, col0: int, w, b, conv_state, seq_first,
 def state_scan(y, src, col_x: int, col_b: int, col_c: int, dt_src,
                col_dt: int, heads: int, groups: int, n_state: int, vdim: int,
                act_silu: bool, dt_bias, a_log, skip, decay, state, seq_first,
-               seq_rows, state_slots, pos32) -> None:
+               seq_rows, state_slots, pos32, single: bool = False) -> None:
+    """`single` (a host-side hint): every sequence brings one row, as in a
+    decode step; the GPU then streams the states through its step kernel."""
     k = _state_backend(src)
     if k is not None:
         k.state_scan(y, src, col_x, col_b, col_c, dt_src, col_dt, heads,
                      groups, n_state, vdim, act_silu, dt_bias, a_log, skip,
-                     decay, state, seq_first, seq_rows, state_slots, pos32)
+                     decay, state, seq_first, seq_rows, state_slots, pos32,
+                     single)
     else:
         torch_ref.state_scan(y, src, col_x, col_b, col_c, dt_src, col_dt,
                              heads, groups, n_state, vdim, act_silu, dt_bias,

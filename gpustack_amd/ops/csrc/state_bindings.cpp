@@ -13,7 +13,7 @@ void head_norm_store_launch(void*, void*, long, int, int, int, const float*, con
 void value_page_store_launch(const void*, long, int, void*, const long*, long, const int*, int, int, int, int, int, hipStream_t);
 void route_topk_launch(int*, float*, const float*, int, const float*, int, int, int, int, int, int, int, int, float, hipStream_t);
 void causal_conv_silu_launch(void*, const void*, long, int, int, int, const float*, const float*, void*, const int*, const int*, const int*, const int*, const int*, int, int, int, int, hipStream_t);
-int state_scan_launch(float*, const void*, long, int, int, int, const void*, long, int, int, int, int, int, int, const float*, const float*, const float*, const float*, float*, const int*, const int*, const int*, const int*, int, int, int, int, hipStream_t);
+int state_scan_launch(float*, const void*, long, int, int, int, const void*, long, int, int, int, int, int, int, const float*, const float*, const float*, const float*, float*, const int*, const int*, const int*, const int*, int, int, int, int, int, hipStream_t);
 void gated_group_norm_launch(void*, const float*, const void*, long, const float*, int, int, int, float, int, int, int, hipStream_t);
 int state_scan_max_state();
 int conv_max_taps();
@@ -243,7 +243,7 @@ void state_scan(Tensor y, Tensor src, long col_x, long col_b, long col_c,
                 long n_state, long vdim, bool act_silu, OptTensor dt_bias,
                 OptTensor a_log, OptTensor skip, OptTensor decay, Tensor state,
                 Tensor seq_first, Tensor seq_rows, Tensor state_slots,
-                Tensor pos32) {
+                Tensor pos32, bool single) {
   chk(y, "y", at::kFloat);
   chk(state, "state", at::kFloat);
   const int bf = view_kind(src, "src");
@@ -290,7 +290,8 @@ void state_scan(Tensor y, Tensor src, long col_x, long col_b, long col_c,
       (int)n_state, (int)vdim, act_silu ? 1 : 0, bp, ap, sp, dp,
       state.data_ptr<float>(), seq_first.data_ptr<int>(),
       seq_rows.data_ptr<int>(), state_slots.data_ptr<int>(),
-      pos32.data_ptr<int>(), nseq, (int)state.size(0), T, bf, cur_stream(src));
+      pos32.data_ptr<int>(), nseq, (int)state.size(0), T, bf, single ? 1 : 0,
+      cur_stream(src));
   TORCH_CHECK(ok, "state size unsupported");
   HIP_CHECK_LAST();
 }

@@ -438,6 +438,84 @@ __global__ __launch_bounds__(256) void state_scan_vec_kernel(
   }
 }
 
+// Single rows (decode): the state itself is the traffic, so one workgroup
+// per (sequence, head) streams it once with 16-byte accesses — a lane
+// owns 4 neighbouring value channels of every RP-th state row — updates it
+// in place and reduces y over the rows through LDS. More rows of a
+// sequence, should a batch bring them, are walked one after the other.
+template <typename TS>
+__global__ __launch_bounds__(256) void state_step_kernel(
+    float* __restrict__ y, const TS* __restrict__ src,
+    const TS* __restrict__ dt_src, ScanArgs p) {
+  extern __shared__ __attribute__((aligned(16))) float sm[];
+  const int N = p.N, P = p.P, P4 = P / 4, RP = 256 / P4;
+  float* vs = sm;                 // [P]      (16-byte reads: P % 4 == 0)
+  float* part = vs + P;           // [RP][P]
+  float* ks = part + RP * P;      // [N]
+  float* qs = ks + N;             // [N]
+  __shared__ float ab[2];
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int cg = tid % P4, r0 = tid / P4;
+  const int first = p.seq_first[s], n = p.seq_rows[s];
+  if (first < 0 || n < 1 || first + n > p.T) return;
+  const int slot = min(max(p.state_slots[s], 0), p.nslots - 1);
+  const int hist = p.pos32[first];
+  const int g = h / (p.H / p.G);
+  float* sp = p.state + ((long)slot * p.H + h) * N * P;
+  const float skip = p.skip != nullptr ? p.skip[h] : 0.f;
+  for (int r = 0; r < n; ++r) {
+    const TS* rp = src + (long)(first + r) * p.ld_src;
+    __syncthreads();
+    for (int i = tid; i < N; i += 256) {
+      float kv = ld(rp + p.col_b + g * N + i), qv = ld(rp + p.col_c + g * N + i);
+      if (p.act) { kv = silu_f(kv); qv = silu_f(qv); }
+      ks[i] = kv;
+      qs[i] = qv;
+    }
+    for (int i = tid; i < P; i += 256) {
+      float v = ld(rp + p.col_x + h * P + i);
+      vs[i] = p.act ? silu_f(v) : v;
+    }
+    if (tid == 0) {
+      if (dt_src != nullptr) {
+        const float dt = softplus_f(
+            ld(dt_src + (long)(first + r) * p.ld_dt + p.col_dt + h) + p.dt_bias[h]);
+        ab[0] = expf(-expf(p.a_log[h]) * dt);
+        ab[1] = dt;
+      } else {
+        ab[0] = p.decay[h];
+        ab[1] = 1.f;
+      }
+    }
+    __syncthreads();
+    const float a = ab[0], b = ab[1];
+    const bool fresh = hist <= 0 && r == 0;      // start from a zero state
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    if (r0 < RP) {
+      const f32x4 v4 = *reinterpret_cast<const f32x4*>(vs + cg * 4);
+      for (int nn = r0; nn < N; nn += RP) {
+        f32x4* at = reinterpret_cast<f32x4*>(sp + (long)nn * P + cg * 4);
+        f32x4 S = fresh ? f32x4{0.f, 0.f, 0.f, 0.f} : *at;
+        const float bk = b * ks[nn], qn = qs[nn];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          S[k] = a * S[k] + bk * v4[k];
+          acc[k] += S[k] * qn;
+        }
+        *at = S;
+      }
+      *reinterpret_cast<f32x4*>(part + r0 * P + cg * 4) = acc;
+    }
+    __syncthreads();
+    for (int i = tid; i < P; i += 256) {
+      float o = skip * vs[i];
+      for (int k = 0; k < RP; ++k) o += part[k * P + i];
+      y[(long)(first + r) * p.H * P + h * P + i] = o;
+    }
+  }
+}
+
 constexpr int ROW_THREADS = 256;
 
 DEVICE_INLINE float block_sum(float v, float* red) {
@@ -626,8 +704,9 @@ void causal_conv_silu_launch(void* out, const void* src, long ld_src, int col0,
   }
 }
 
-// src_bf: src and dt_src are bf16 (else fp32). Returns 0 when no
-// instantiation covers the sizes.
+// src_bf: src and dt_src are bf16 (else fp32). single: the caller expects
+// one row per sequence (a hint: any batch is still computed correctly).
+// Returns 0 when no instantiation covers the sizes.
 int state_scan_launch(float* y, const void* src, long ld_src, int col_x,
                       int col_b, int col_c, const void* dt_src, long ld_dt,
                       int col_dt, int H, int G, int N, int P, int act,
@@ -635,7 +714,8 @@ int state_scan_launch(float* y, const void* src, long ld_src, int col_x,
                       const float* skip, const float* decay, float* state,
                       const int* seq_first, const int* seq_rows,
                       const int* state_slots, const int* pos32, int nseq,
-                      int nslots, int T, int src_bf, hipStream_t s) {
+                      int nslots, int T, int src_bf, int single,
+                      hipStream_t s) {
   if (T <= 0 || nseq <= 0) return 1;
   ScanArgs p;
   p.ld_src = ld_src; p.ld_dt = ld_dt; p.col_x = col_x; p.col_b = col_b;
@@ -644,6 +724,20 @@ int state_scan_launch(float* y, const void* src, long ld_src, int col_x,
   p.decay = decay; p.state = state; p.seq_first = seq_first;
   p.seq_rows = seq_rows; p.state_slots = state_slots; p.pos32 = pos32;
   p.nslots = nslots; p.T = T;
+  // batches of single rows: the streaming step kernel, when the value size
+  // splits a workgroup evenly into 16-byte columns
+  const int P4 = P / 4;
+  if (single && P % 4 == 0 && P4 >= 1 && P4 <= 256 && 256 % P4 == 0 &&
+      (size_t)(2 * N + P + (256 / P4) * P) * sizeof(float) <= 48 * 1024) {
+    const size_t smem = (size_t)(2 * N + P + (256 / P4) * P) * sizeof(float);
+    if (src_bf)
+      state_step_kernel<unsigned short><<<dim3(nseq, H), 256, smem, s>>>(
+          y, (const unsigned short*)src, (const unsigned short*)dt_src, p);
+    else
+      state_step_kernel<float><<<dim3(nseq, H), 256, smem, s>>>(
+          y, (const float*)src, (const float*)dt_src, p);
+    return 1;
+  }
   if (src_bf)
     return scan_pick<unsigned short, unsigned short>(y, src, dt_src, p, nseq, s);
   return scan_pick<float, float>(y, src, dt_src, p, nseq, s);

@@ -190,17 +190,21 @@ def test_state_scan(dtype, H, G, N, P, stepped, off):
     else:
         decay = torch.linspace(0.5, 0.999, H, device=DEV)
         extra = (None, 0, H, G, N, P, True, None, None, None, decay)
-    res = []
-    for impl in (ops, torch_ref):
+    def run(impl, **kw):
         y = torch.zeros(T, H * P, device=DEV)
         st = st0.clone()
-        impl.state_scan(y, src, cx, cb, cc, *extra, st, sf, sr, ss, pos)
-        res.append((y, st))
-    scale = res[1][0].abs().max().clamp(min=1.0)
-    assert (res[0][0] - res[1][0]).abs().max() <= 2e-4 * scale
-    sscale = res[1][1].abs().max().clamp(min=1.0)
-    assert (res[0][1] - res[1][1]).abs().max() <= 2e-4 * sscale
-    assert torch.equal(res[0][1][6], st0[6])
+        impl.state_scan(y, src, cx, cb, cc, *extra, st, sf, sr, ss, pos, **kw)
+        return y, st
+
+    ry, rst = run(torch_ref)
+    scale = ry.abs().max().clamp(min=1.0)
+    sscale = rst.abs().max().clamp(min=1.0)
+    # the scan kernels, and the decode step kernel on the same ragged batch
+    for kw in ({}, {"single": True}):
+        y, st = run(ops, **kw)
+        assert (y - ry).abs().max() <= 2e-4 * scale, kw
+        assert (st - rst).abs().max() <= 2e-4 * sscale, kw
+        assert torch.equal(st[6], st0[6])
 
 
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
