@@ -21,26 +21,68 @@ class LatentMixerSpec:
     v_dim: int
     kv_rank: int
     scale: float
+    # the rotary variant (models/latent_attention.py RotaryLatentAttention):
+    # rot_dim > 0 adds a rotated part to every query head and ONE rotated
+    # key part per token shared by all heads, cached beside the latent;
+    # q_rank > 0 sends the queries through a normed latent of their own;
+    # window > 0: a row sees the last `window` positions, itself included;
+    # sink: a learned logit per head joins the softmax denominator;
+    # out_gate: each head's output times a sigmoid gate read from the
+    # mixer's input; kv_from >= 0: no down-projection and no pool of its
+    # own — the layer reads the latent and rotated key part that layer
+    # `kv_from` cached
+    rot_dim: int = 0
+    rot: "RotarySpec | None" = None
+    q_rank: int = 0
+    window: int = 0
+    sink: bool = False
+    out_gate: bool = False
+    kv_from: int = -1
 
 
 @dataclass(frozen=True)
 class RotarySpec:
-    """Pairwise rotary positions on the first `dims` channels of a head:
-    channel 2i pairs with 2i+1 and turns by pos * f_i, f_i = base^(-2i/dims),
-    optionally with wavelength-dependent frequency scaling (`scaling`:
-    factor / low / high / original — long waves slowed by `factor`, short
-    ones kept, a linear blend between)."""
+    """Rotary positions on the first `dims` channels of a head, the pair i
+    turning by pos * f_i, f_i = base^(-2i/dims). `layout` "pairs": channel
+    2i pairs with 2i+1; "half": channel i pairs with i + dims/2. Optional
+    wavelength-dependent frequency scaling, one of
+    * `scaling` (factor, low, high, original): long waves slowed by
+      `factor`, short ones kept, a linear blend in the wavelength between;
+    * `ramp` (factor, original, fast, slow): the blend is linear in the
+      CHANNEL index between the channels that make `fast` and `slow` turns
+      over `original` positions, and cos / sin are multiplied by
+      `amplitude` = 0.1 ln(factor) + 1."""
     dims: int = 0
     base: float = 10000.0
     scaling: tuple | None = None        # (factor, low, high, original)
+    layout: str = "pairs"               # "pairs" | "half"
+    ramp: tuple | None = None           # (factor, original, fast, slow)
+
+    @property
+    def amplitude(self) -> float:
+        import math
+
+        return 0.1 * math.log(self.ramp[0]) + 1.0 if self.ramp else 1.0
 
     def inv_freq(self) -> list[float]:
         """f_i for i < dims/2, in double precision."""
         import math
 
         out = []
+        if self.ramp is not None:
+            factor, orig, fast, slow = self.ramp
+
+            def chan(turns):
+                return (self.dims * math.log(orig / (2.0 * math.pi * turns))
+                        / (2.0 * math.log(self.base)))
+
+            lo = max(math.floor(chan(fast)), 0)
+            hi = min(math.ceil(chan(slow)), self.dims - 1)
         for i in range(self.dims // 2):
             f = self.base ** (-2.0 * i / self.dims)
+            if self.ramp is not None:
+                r = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+                f = f / factor * r + f * (1.0 - r)
             if self.scaling is not None:
                 factor, low, high, orig = self.scaling
                 wave = 2.0 * math.pi / f
@@ -77,7 +119,10 @@ class PagedMixerSpec:
       query i and key j, slope_h = 2^(-8 (h + 1) / heads).
     * v_mix: the layer's values blend with the values the FIRST such layer
       of the stack computed for the same token, v <- (1 - l) v + l v_first
-      with one learned l per layer; the blend is what the pool keeps."""
+      with one learned l per layer; the blend is what the pool keeps.
+    * softcap > 0: the scaled score s becomes softcap * tanh(s / softcap).
+    * head_norm together with a rotation (rot.dims > 0) and biases: the
+      per-head norm comes first, then the rotation."""
     heads: int
     kv_heads: int
     qk_dim: int
@@ -96,6 +141,7 @@ class PagedMixerSpec:
     q_temp: tuple | None = None         # (coef, every)
     distance_bias: bool = False
     v_mix: bool = False
+    softcap: float = 0.0
 
     def slopes(self) -> list[float]:
         """Distance-bias slope of every head, in double precision."""
@@ -125,7 +171,14 @@ class ScanMixerSpec:
       is gated by silu(z), then RMS-normed in `norm_groups` parts.
     * kind "lightning": a_t = decay[h] (constants), b_t = 1, q / k / v are
       SiLU of their projections (one k and q per head); the output is
-      RMS-normed over all heads, then multiplied by a sigmoid gate."""
+      RMS-normed over all heads, then multiplied by a sigmoid gate.
+    * kind "delta" (gated delta rule): S <- g_t S; u = beta_t (v_t - S^T
+      k_t); S <- S + k_t u^T; y_t = S^T q_t with g_t = exp(-exp(A_log) *
+      softplus(a_t + dt_bias)) and beta_t = sigmoid(b_t) per head and token;
+      q, k (shared by the heads of a group) and v pass a causal convolution
+      of `conv` taps and SiLU, then q and k are scaled to unit length (q
+      also by state^(-1/2)); each head's output is RMS-normed, weighted and
+      multiplied by a SiLU gate."""
     kind: str
     heads: int
     state: int                          # rows of the state = size of k and q
@@ -142,6 +195,16 @@ class ScanMixerSpec:
     @property
     def conv_channels(self) -> int:     # x | B | C
         return (self.inner + 2 * self.groups * self.state) if self.conv else 0
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """Two mixers side by side on the same input (models/parallel_mixer.py):
+    softmax attention over the paged pool and a recurrent matrix-state
+    mixer; each output is RMS-normed over the model width with its own
+    weight and the two are averaged."""
+    left: PagedMixerSpec
+    right: ScanMixerSpec
 
 
 @dataclass(frozen=True)
@@ -177,8 +240,9 @@ class FeedForwardSpec:
 @dataclass(frozen=True)
 class LayerSpec:
     """One entry of a heterogeneous layer stack (ModelSpec.layers)."""
-    mixer_type: str         # "latent_attention" | "paged_attention" | "scan"
-    mixer: "LatentMixerSpec | PagedMixerSpec | ScanMixerSpec"
+    # "latent_attention" | "paged_attention" | "scan" | "parallel"
+    mixer_type: str
+    mixer: "LatentMixerSpec | PagedMixerSpec | ScanMixerSpec | ParallelMixerSpec"
     mlp: FeedForwardSpec | None = None
 
 
@@ -303,6 +367,8 @@ class ModelSpec:
     # pass with cache pools of its own; each pass but the first starts by
     # adding the embedding output to the stream. None = every layer once
     layer_loop: tuple | None = None      # (start, stop, times)
+    # the embedding output passes a norm of its own before the first layer
+    embed_norm: bool = False
 
     @property
     def gqa_ratio(self) -> int:
@@ -322,13 +388,24 @@ class ModelSpec:
         return runs + [(i, False) for i in range(stop, n)]
 
     def kv_pool_widths(self) -> list[tuple]:
-        """Per layer run of a heterogeneous stack: ("latent", rank) or
-        ("kv", kv_heads, key width, value width)."""
+        """Per layer run of a heterogeneous stack: ("latent", rank),
+        ("kv", kv_heads, key width, value width), ("state",) for a run that
+        keeps nothing per token, or ("shared", run) for a run that reads
+        the pools of an earlier one."""
         out = []
         for i, _ in self.layer_runs():
             m = self.layers[i].mixer
+            if isinstance(m, ParallelMixerSpec):
+                m = m.left
             if isinstance(m, LatentMixerSpec):
-                out.append(("latent", m.kv_rank))
+                if m.kv_from >= 0:
+                    out.append(("shared", m.kv_from))
+                elif m.rot_dim:
+                    # one key "head" per token: latent | rotated key part;
+                    # the latent again, page-transposed, as the value
+                    out.append(("kv", 1, m.kv_rank + m.rot_dim, m.kv_rank))
+                else:
+                    out.append(("latent", m.kv_rank))
             elif isinstance(m, ScanMixerSpec):
                 out.append(("state",))      # nothing per token: a state slot
             else:
@@ -341,6 +418,8 @@ class ModelSpec:
         out = []
         for i, _ in self.layer_runs():
             m = self.layers[i].mixer
+            if isinstance(m, ParallelMixerSpec):
+                m = m.right
             if isinstance(m, ScanMixerSpec):
                 out.append((m.heads, m.state, m.vdim,
                             max(m.conv - 1, 0), m.conv_channels))
@@ -360,12 +439,14 @@ class ModelSpec:
     @property
     def has_state(self) -> bool:
         return self.layers is not None and any(
-            isinstance(ls.mixer, ScanMixerSpec) for ls in self.layers)
+            isinstance(ls.mixer, (ScanMixerSpec, ParallelMixerSpec))
+            for ls in self.layers)
 
     def kv_bytes_per_token(self, dtype_size: int = 2) -> int:
         if self.layers is not None:
             return sum(w[1] if w[0] == "latent" else
-                       0 if w[0] == "state" else w[1] * (w[2] + w[3])
+                       0 if w[0] in ("state", "shared")
+                       else w[1] * (w[2] + w[3])
                        for w in self.kv_pool_widths()) * dtype_size
         if self.kv_lora_rank:
             # MLA: one compressed latent row per token per layer
@@ -382,6 +463,11 @@ class ModelSpec:
                 n += (self.bigram_buckets + 1) * h
             for ls in self.layers:
                 m = ls.mixer
+                if self.architecture == "Makezen":
+                    n += self._mixer_weights(h, m) + 2 * h
+                    if ls.mlp is not None:
+                        n += 2 * h * ls.mlp.ff + 2 * h
+                    continue
                 if isinstance(m, ScanMixerSpec):
                     if m.kind == "mamba2":
                         n += (h * (2 * m.inner + 2 * m.groups * m.state
@@ -450,6 +536,29 @@ class ModelSpec:
             total_layers = (attn_norm + dense_mlp) * self.num_layers
         emb = v * h * (1 if self.tie_word_embeddings else 2)
         return (total_layers + emb + h) * dtype_size
+
+    @classmethod
+    def _mixer_weights(cls, h: int, m) -> int:
+        """Weight count of one mixer of a Makezen stack."""
+        if isinstance(m, ParallelMixerSpec):
+            return (cls._mixer_weights(h, m.left)
+                    + cls._mixer_weights(h, m.right) + 2 * h)
+        if isinstance(m, ScanMixerSpec):        # gated delta rule
+            qk = 2 * m.groups * m.state
+            return (h * (qk + 2 * m.inner + 2 * m.heads)
+                    + (qk + m.inner) * m.conv + 2 * m.heads + m.vdim
+                    + m.inner * h)
+        if isinstance(m, PagedMixerSpec):
+            return ((h + 1) * (m.qk_dim * (m.heads + m.kv_heads)
+                               + m.kv_heads * m.v_dim)
+                    + 2 * m.qk_dim + m.heads * m.v_dim * h)
+        qd = m.qk_dim + m.rot_dim
+        n = (h * m.q_rank + m.q_rank + m.q_rank * m.heads * qd
+             + m.kv_rank * m.heads * (m.qk_dim + m.v_dim)
+             + 2 * m.heads + m.heads * h + m.heads * m.v_dim * h)
+        if m.kv_from < 0:
+            n += h * (m.kv_rank + m.rot_dim) + m.kv_rank
+        return n
 
     @staticmethod
     def _rope_scaling_from(cfg: dict) -> dict | None:
@@ -698,7 +807,112 @@ class ModelSpec:
         )
 
     @classmethod
+    def _from_makezen_config(cls, cfg: dict) -> "ModelSpec":
+        """Makezen checkpoints list their layers one by one; an entry names
+        its mixer — "latent_attention" (rotary latent attention behind a
+        sliding window, with sinks, an output gate and optionally the
+        cached latents of an earlier layer), "delta" (gated delta rule) or
+        "parallel" (softmax attention and a gated delta rule side by side)
+        — and an ungated dense feed-forward or none. Every sublayer sits
+        between two weight-only layer norms on an fp32 stream; the
+        embedding output is normed and the head is the embedding table."""
+        def rotary(r):
+            if not r or not int(r.get("dims", 0) or 0):
+                return RotarySpec(layout="half")
+            sc = r.get("scaling") or None
+            return RotarySpec(
+                dims=int(r["dims"]), base=float(r["base"]), layout="half",
+                ramp=(float(sc["factor"]), float(sc["original"]),
+                      float(sc["fast"]), float(sc["slow"])) if sc else None)
+
+        def delta(m):
+            sp = ScanMixerSpec(
+                kind="delta", heads=int(m["heads"]), state=int(m["dim"]),
+                vdim=int(m["vdim"]), groups=int(m["kv_heads"]),
+                conv=int(m["conv"]))
+            if sp.heads % sp.groups or sp.conv < 1:
+                raise ValueError("delta mixer sizes do not divide")
+            return sp
+
+        def softmax(m):
+            sp = PagedMixerSpec(
+                heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
+                qk_dim=int(m["dim"]), v_dim=int(m.get("vdim", m["dim"])),
+                scale=float(m["scale"]), rot=rotary(m.get("rot")), bias=True,
+                head_norm=True, softcap=float(m.get("softcap") or 0.0),
+                window=int((m.get("mask") or {}).get("size", 0) or 0))
+            if sp.heads % sp.kv_heads:
+                raise ValueError("heads must be a multiple of kv_heads")
+            if sp.rot.dims % 2 or sp.rot.dims > sp.qk_dim:
+                raise ValueError("rotary dims must be even and fit the head")
+            return sp
+
+        layers = []
+        for i, ent in enumerate(cfg["layers"]):
+            m, kind = ent["mixer"], ent["type"]
+            if kind == "latent_attention":
+                rot = rotary(m.get("rot"))
+                src = m.get("kv_from")
+                mixer = LatentMixerSpec(
+                    heads=int(m["heads"]), qk_dim=int(m["dim"]),
+                    v_dim=int(m["vdim"]), kv_rank=int(m["kv_rank"]),
+                    scale=float(m["scale"]), rot_dim=int(m["rot_dim"]),
+                    rot=rot, q_rank=int(m["q_rank"]),
+                    window=int((m.get("mask") or {}).get("size", 0) or 0),
+                    sink=True, out_gate=True,
+                    kv_from=-1 if src is None else int(src))
+                if rot.dims != mixer.rot_dim or rot.dims % 2 or not rot.dims:
+                    raise ValueError("the rotated part is rot_dim wide")
+                if mixer.kv_from >= 0:
+                    own = layers[mixer.kv_from].mixer \
+                        if mixer.kv_from < i else None
+                    if not isinstance(own, LatentMixerSpec) \
+                            or own.kv_from >= 0 \
+                            or (own.kv_rank, own.rot_dim, own.rot) != (
+                                mixer.kv_rank, mixer.rot_dim, mixer.rot):
+                        raise ValueError(
+                            "kv_from must name an earlier latent layer with "
+                            "its own down-projection and the same latent "
+                            "sizes and rotation")
+                mtype = "latent_attention"
+            elif kind == "delta":
+                mixer, mtype = delta(m), "scan"
+            elif kind == "parallel":
+                mixer = ParallelMixerSpec(left=softmax(m["left"]),
+                                          right=delta(m["right"]))
+                mtype = "parallel"
+            else:
+                raise NotImplementedError(
+                    f"Makezen mixer type {kind!r} is not implemented")
+            f = ent.get("mlp")
+            if not f:
+                ff = None
+            elif f["kind"] == "dense":
+                ff = FeedForwardSpec(kind="dense", ff=int(f["ff"]),
+                                     act="gelu_tanh")
+            else:
+                raise NotImplementedError(
+                    f"Makezen feed-forward kind {f['kind']!r}")
+            layers.append(LayerSpec(mtype, mixer, ff))
+        return cls(
+            architecture="Makezen",
+            vocab_size=int(cfg["vocab"]),
+            hidden_size=int(cfg["width"]),
+            num_layers=len(layers),
+            layers=tuple(layers),
+            num_heads=1, num_kv_heads=1, head_dim=8, intermediate_size=0,
+            rms_norm_eps=float(cfg["norm"]["eps"]),
+            max_position_embeddings=int(
+                cfg.get("max_position_embeddings", 1 << 20)),
+            eos_token_id=int(cfg.get("eos_token_id", -1)),
+            sandwich_norms=True, fp32_residual=True, norm_type="layernorm",
+            embed_norm=True, tie_word_embeddings=True,
+        )
+
+    @classmethod
     def from_hf_config(cls, cfg: dict) -> "ModelSpec":
+        if cfg.get("architecture") == "Makezen" and "architectures" not in cfg:
+            return cls._from_makezen_config(cfg)
         if cfg.get("architecture") == "Livasun" and "architectures" not in cfg:
             return cls._from_livasun_config(cfg)
         if cfg.get("architecture") == "Vunitar" and "architectures" not in cfg:

@@ -213,6 +213,11 @@ class KVCache:
             self.num_layers = len(widths)
             self.k_caches, self.v_caches = [], []
             for w in widths:
+                if w[0] == "shared":
+                    # the run reads (never writes) an earlier run's pools
+                    self.k_caches.append(self.k_caches[w[1]])
+                    self.v_caches.append(self.v_caches[w[1]])
+                    continue
                 if w[0] == "state":
                     ks = vs = (0,)
                 elif w[0] == "latent":
@@ -381,7 +386,7 @@ class KVCache:
             planes = KVCache.latent_planes(cfg)
             per_block = max(1, cfg.block_size * esize * sum(
                 w[1] * planes if w[0] == "latent" else
-                0 if w[0] == "state" else w[1] * (w[2] + w[3])
+                0 if w[0] in ("state", "shared") else w[1] * (w[2] + w[3])
                 for w in spec.kv_pool_widths()))
         elif spec.kv_lora_rank:
             per_block = (nl * cfg.block_size

@@ -6,6 +6,7 @@ _MODEL_CLASSES = {
     "Vunitar": ("vunitar", "VunitarForCausalLM"),
     "Fusipel": ("fusipel", "FusipelForCausalLM"),
     "Livasun": ("livasun", "LivasunForCausalLM"),
+    "Makezen": ("makezen", "MakezenForCausalLM"),
 }
 
 

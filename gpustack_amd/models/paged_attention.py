@@ -17,7 +17,10 @@ variants, every one a parameter of PagedMixerSpec:
   a query temperature growing with the logarithm of the position, a
   per-head slope times the distance taken off every score, and values
   blended with those the first such layer of the stack computed for the
-  same token (ops.head_norm_store prepares q and writes the pool).
+  same token (ops.head_norm_store prepares q and writes the pool);
+* the per-head q / k norm FOLLOWED by a rotation (either pairing layout,
+  optionally with a cos / sin amplitude) and with projection biases
+  (ops.head_rope_store), and a tanh cap on the scaled scores.
 
 Flow per step: one fused q/k/v GEMM -> ops.rotary_norm_store (norm, rotary,
 cache write, all fp32 inside) -> ops.paged_attention over the block tables
@@ -41,11 +44,20 @@ class PagedRotaryAttention(nn.Module):
     def __init__(self, width: int, m: PagedMixerSpec, eps: float, dtype,
                  comm=None, v_mix_first: bool = False):
         super().__init__()
-        if m.head_norm and (m.rot.dims or m.qk_norm_full or m.tied_values
-                            or m.maps != 1 or m.bias):
+        # per-head norm, then rotation: the generic per-head row kernel
+        self.rope_rows = bool(m.head_norm and (m.rot.dims or m.bias)) \
+            or m.rot.layout == "half"
+        if self.rope_rows and (m.qk_norm_full or m.tied_values or m.maps != 1
+                               or m.q_temp or m.v_mix or m.distance_bias):
             raise NotImplementedError(
-                "per-head q/k norm is served without rotation, biases, "
-                "whole-row norms, tied values or a second score map")
+                "the per-head norm + rotation row kernel serves one score "
+                "map with its own values, without whole-row norms, query "
+                "temperature, distance bias or value mixing")
+        if m.head_norm and not self.rope_rows and (
+                m.qk_norm_full or m.tied_values or m.maps != 1):
+            raise NotImplementedError(
+                "per-head q/k norm is served without whole-row norms, tied "
+                "values or a second score map")
         if (m.q_temp or m.v_mix) and not m.head_norm:
             raise NotImplementedError(
                 "query temperature and value mixing come with the per-head "
@@ -109,7 +121,15 @@ class PagedRotaryAttention(nn.Module):
         q = torch.empty(T, self.nq, dtype=h.dtype, device=h.device)
         groups = (rg.page_groups(k_cache.shape[2])
                   if h.is_cuda and k_cache.shape[2] == 16 else None)
-        if m.head_norm:
+        if self.rope_rows:
+            rot0 = 0 if m.rot.dims else -1
+            ops.head_rope_store(
+                q, qkv, 0, m.heads, m.qk_dim, self.q_head_norm, m.qk_dim,
+                rot0, self.nq, m.kv_heads, m.qk_dim, self.k_head_norm,
+                m.qk_dim, rot0, self.nq + self.nk, self.inv_freq,
+                m.rot.layout == "half", m.rot.amplitude, rg.pos32, k_cache,
+                v_cache, meta.slot_mapping, self.eps, page_groups=groups)
+        elif m.head_norm:
             v_first = None
             if m.v_mix and not self.v_mix_first:
                 v_first = shared["v_first"]
@@ -136,7 +156,8 @@ class PagedRotaryAttention(nn.Module):
             rg.row_seq, rg.pos32, m.scale, maps=m.maps, window=m.window,
             keep_first=m.keep_first, sinks=self.sinks,
             tiles=rg.attn_tiles(m.heads, m.kv_heads, m.maps) if h.is_cuda
-            else None, max_ctx=rg.max_ctx, slopes=self.slopes)
+            else None, max_ctx=rg.max_ctx, slopes=self.slopes,
+            softcap=m.softcap)
         if m.maps == 2:
             o = torch.empty(T, m.heads * self.vw, dtype=h.dtype,
                             device=h.device)

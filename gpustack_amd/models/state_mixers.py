@@ -20,6 +20,14 @@ states. Nothing is kept per token.
   SiLU on their way into the scan; a_t is a constant per head, b_t = 1. The
   output is RMS-normed over all heads and multiplied by sigmoid(g).
 
+* GatedDeltaMixer runs the gated delta rule instead (ops.delta_scan),
+      S_t = g_t S_(t-1) + k_t u_t^T,  u_t = beta_t (v_t - (g_t S_(t-1))^T k_t),
+  y_t = S_t^T q_t: one projection gives q | k | v | gate | a | b; q, k, v
+  pass the convolution and SiLU, q and k are scaled to unit length inside
+  the scan, g_t = exp(-exp(A_log) softplus(a + dt_bias)), beta_t =
+  sigmoid(b); each head's output is RMS-normed, weighted and multiplied by
+  silu(gate).
+
 Decays, step sizes, the recurrence and both norms are fp32; the
 projections (library GEMMs) and the convolution run in the engine dtype.
 """
@@ -117,8 +125,60 @@ class LightningMixer(nn.Module):
         return self.comm.all_reduce(out) if self.comm is not None else out
 
 
+class GatedDeltaMixer(nn.Module):
+    def __init__(self, width: int, m: ScanMixerSpec, eps: float, dtype,
+                 comm=None):
+        super().__init__()
+        if comm is not None and comm.tp_size > 1:
+            raise NotImplementedError(
+                "recurrent mixers are not sharded for tensor parallelism yet")
+        self.m, self.eps, self.comm = m, eps, comm
+        f32 = torch.float32
+        self.nqk = m.groups * m.state
+        # columns of the projection: q | k | v | gate | a | b
+        self.col_gate = 2 * self.nqk + m.inner
+        self.col_a = self.col_gate + m.inner
+        self.col_b = self.col_a + m.heads
+        self.in_w = _mk(self.col_b + m.heads, width, dt=dtype)
+        self.conv_w = _mk(m.conv_channels, m.conv, dt=f32)   # q | k | v
+        self.register_buffer("conv_b", torch.zeros(m.conv_channels, dtype=f32),
+                             persistent=False)
+        self.dt_bias = _mk(m.heads, dt=f32)
+        self.a_log = _mk(m.heads, dt=f32)
+        self.norm = _mk(m.vdim, dt=f32)          # one weight vector, all heads
+        self.register_buffer("norm_rows", torch.ones(m.inner, dtype=f32),
+                             persistent=False)
+        self.o_w = _mk(width, m.inner, dt=dtype)
+
+    def post_load(self) -> None:
+        self.norm_rows.copy_(self.norm.repeat(self.m.heads))
+
+    def forward(self, h, meta, ssm_state, conv_state):
+        m = self.m
+        rg = meta.ragged
+        T = h.shape[0]
+        u = F.linear(h, self.in_w)
+        qkv = torch.empty(T, m.conv_channels, dtype=h.dtype, device=h.device)
+        ops.causal_conv_silu(qkv, u, 0, self.conv_w, self.conv_b, conv_state,
+                             rg.seq_first, rg.seq_rows, rg.state_slots,
+                             rg.row_seq, rg.pos32)
+        y = torch.empty(T, m.inner, dtype=torch.float32, device=h.device)
+        ops.delta_scan(y, qkv, 0, self.nqk, 2 * self.nqk, u, self.col_a,
+                       self.col_b, m.heads, m.groups, m.state, m.vdim,
+                       self.dt_bias, self.a_log, ssm_state, rg.seq_first,
+                       rg.seq_rows, rg.state_slots, rg.pos32,
+                       single=max(rg.seq_news, default=1) <= 1)
+        g = torch.empty(T, m.inner, dtype=h.dtype, device=h.device)
+        ops.gated_group_norm(g, y, u[:, self.col_gate:self.col_a],
+                             self.norm_rows, m.heads, self.eps, 2)
+        out = F.linear(g, self.o_w)
+        return self.comm.all_reduce(out) if self.comm is not None else out
+
+
 def build_scan_mixer(width: int, m: ScanMixerSpec, eps: float, dtype,
                      comm=None):
+    if m.kind == "delta":
+        return GatedDeltaMixer(width, m, eps, dtype, comm)
     if m.kind == "mamba2":
         return Mamba2Mixer(width, m, eps, dtype, comm)
     if m.kind == "lightning":

@@ -59,12 +59,18 @@ def _layered_tensor_plan(model):
     plan.append(("embed", model.embed, same))
     if getattr(model, "pair_table", None) is not None:
         plan.append(("bigram", model.pair_table, same))
+    if getattr(model, "embed_norm", None) is not None:
+        plan.append(("embed.norm", model.embed_norm, same))
     plan.append(("final.norm", model.final_norm, same))
     if getattr(model, "final_norm_b", None) is not None:
         plan.append(("final.norm.b", model.final_norm_b, same))
-    plan.append(("head", model.lm_head, same))
+    if not getattr(model, "tied_head", False):
+        plan.append(("head", model.lm_head, same))
     for i, layer in enumerate(model.layers):
         p = f"l{i}."
+        if hasattr(layer, "mixer") and hasattr(layer, "pre1"):
+            plan += _sandwich_ln_layer_plan(p, layer)
+            continue
         if hasattr(layer, "mixer"):
             plan += _prenorm_layer_plan(p, layer)
             continue
@@ -143,6 +149,102 @@ def _paged_layer_plan(p: str, layer):
                      (p + "mlp.up", m.up_w[m.ff:], same)]
         else:
             plan.append((p + "mlp.up", m.up_w, same))
+    return plan
+
+
+def _shaped(fn, *src_shape):
+    """A layout transform that also tells the shape of the checkpoint
+    tensor it expects (random init generates in that shape)."""
+    def wrapped(t):
+        return fn(t)
+
+    wrapped.src_shape = tuple(src_shape)
+    return wrapped
+
+
+def _delta_mixer_plan(p: str, a):
+    """Plan entries of a gated delta rule mixer (models/state_mixers.py):
+    q | k | v | gate | a | b fuse into one projection, the three
+    convolutions into one weight table."""
+    same = lambda t: t
+    n, i, hd = a.nqk, a.m.inner, a.m.heads
+    return [
+        (p + "q", a.in_w[:n], same), (p + "k", a.in_w[n:2 * n], same),
+        (p + "v", a.in_w[2 * n:2 * n + i], same),
+        (p + "g", a.in_w[a.col_gate:a.col_a], same),
+        (p + "a", a.in_w[a.col_a:a.col_b], same),
+        (p + "b", a.in_w[a.col_b:a.col_b + hd], same),
+        (p + "q.conv", a.conv_w[:n], same),
+        (p + "k.conv", a.conv_w[n:2 * n], same),
+        (p + "v.conv", a.conv_w[2 * n:], same),
+        (p + "A_log", a.a_log, same), (p + "dt_bias", a.dt_bias, same),
+        (p + "norm", a.norm, same), (p + "o", a.o_w, same),
+    ]
+
+
+def _head_norm_attention_plan(p: str, a):
+    """Plan entries of a paged attention mixer with biases and per-head
+    q / k norms (models/paged_attention.py)."""
+    same = lambda t: t
+    nq, nk = a.nq, a.nk
+    return [
+        (p + "q", a.qkv_w[:nq], same), (p + "k", a.qkv_w[nq:nq + nk], same),
+        (p + "v", a.qkv_w[nq + nk:], same),
+        (p + "q.b", a.qkv_b[:nq], same),
+        (p + "k.b", a.qkv_b[nq:nq + nk], same),
+        (p + "v.b", a.qkv_b[nq + nk:], same),
+        (p + "q.norm", a.q_head_norm, same),
+        (p + "k.norm", a.k_head_norm, same), (p + "o", a.o_w, same),
+    ]
+
+
+def _rotary_latent_plan(p: str, a):
+    """Plan entries of a rotary latent attention mixer
+    (models/latent_attention.py): the query latent, the key/value latent
+    with its key part (when the layer owns them) and the head gates fuse
+    into one projection; U_k is stored head-major and extended by the
+    identity block of the rotated part, U_v head-major and transposed."""
+    same = lambda t: t
+    plan = [
+        (p + "dq", a.in_w[:a.qr], same), (p + "dq.norm", a.q_norm, same),
+        (p + "uq", a.uq_w, same),
+        (p + "uk", a.uk_ext, _shaped(a.extend_uk, a.h * a.dq, a.r)),
+        (p + "uv", a.uv_t,
+         _shaped(lambda t, a=a: t.view(a.h, a.dv, a.r).transpose(1, 2),
+                 a.h * a.dv, a.r)),
+        (p + "o", a.o_w, same),
+    ]
+    if a.own_kv:
+        plan += [(p + "dkv", a.in_w[a.qr:a.col_g], same),
+                 (p + "dkv.norm", a.kv_norm, same)]
+    if a.sinks is not None:
+        plan.append((p + "sink", a.sinks, same))
+    if a.m.out_gate:
+        plan.append((p + "g", a.in_w[a.col_g:], same))
+    return plan
+
+
+def _sandwich_ln_layer_plan(p: str, layer):
+    """Plan entries of one layer between weight-only layer norms whose
+    mixer is rotary latent attention, a gated delta rule or both kinds side
+    by side (models/makezen.py), with an ungated dense feed-forward."""
+    same = lambda t: t
+    a = layer.mixer
+    plan = [(p + "norm1", layer.pre1, same), (p + "norm1b", layer.post1, same)]
+    if layer.kind == "latent_attention":
+        plan += _rotary_latent_plan(p + "mix.", a)
+    elif layer.kind == "scan":
+        plan += _delta_mixer_plan(p + "mix.", a)
+    else:
+        plan += _head_norm_attention_plan(p + "mix.left.", a.left)
+        plan += _delta_mixer_plan(p + "mix.right.", a.right)
+        plan += [(p + "mix.left.out", a.left_out, same),
+                 (p + "mix.right.out", a.right_out, same)]
+    m = layer.mlp
+    if m is not None:
+        plan += [(p + "norm2", layer.pre2, same),
+                 (p + "norm2b", layer.post2, same),
+                 (p + "mlp.up", m.up_w, same), (p + "mlp.down", m.down_w, same)]
     return plan
 
 
@@ -238,7 +340,9 @@ def _random_init_layered(model, cfg: EngineConfig) -> None:
             continue
         # generate in the checkpoint's own [out, in] shape, then apply the
         # same layout transform the loader uses
-        if name.endswith("mix.uk"):
+        if getattr(fn, "src_shape", None):
+            a_shape = fn.src_shape
+        elif name.endswith("mix.uk"):
             a_shape = (dst.shape[0] * dst.shape[1], dst.shape[2])
         elif name.endswith("mix.uv"):
             a_shape = (dst.shape[0] * dst.shape[2], dst.shape[1])

@@ -592,12 +592,15 @@ def rms_norm_rows(out, x, weight, eps: float) -> None:
 
 
 def sandwich_add_norm(x, a, post_w, mult: float, eps: float, extra, next_w,
-                      h) -> None:
+                      h, center: bool = False) -> None:
+    """`center`: both norms are weight-only layer norms (the mean comes off
+    first) instead of RMS norms."""
     k = _paged_backend(x)
     if k is not None:
-        k.sandwich_add_norm(x, a, post_w, mult, eps, extra, next_w, h)
+        k.sandwich_add_norm(x, a, post_w, mult, eps, extra, next_w, h, center)
     else:
-        torch_ref.sandwich_add_norm(x, a, post_w, mult, eps, extra, next_w, h)
+        torch_ref.sandwich_add_norm(x, a, post_w, mult, eps, extra, next_w, h,
+                                    center)
 
 
 def build_page_groups(seq_starts, seq_hists, seq_news, block_size: int,
@@ -684,14 +687,15 @@ def paged_attention(out, q, k_cache, v_cache, block_tables, row_seq, positions,
                     scale: float, maps: int = 1, window: int = 0,
                     keep_first: int = 0, sinks=None, tiles=None,
                     exact: bool = False, max_ctx: int = 0,
-                    slopes=None) -> None:
-    """q: [T, A, D], out: [T, A, VW] (A = heads * maps score maps). On the
+                    slopes=None, softcap: float = 0.0) -> None:
+    """q: [T, A, D], out: [T, A, VW] (A = heads * maps score maps; views
+    whose last axis is contiguous). On the
     GPU the MFMA kernel runs for bf16 pools of fitting sizes, the fp32
     vector-ALU kernel otherwise (always for fp32 pools, or with `exact`).
     `max_ctx` (longest context in the batch, a host number) lets a batch of
     few tiles over long contexts split each tile's keys over workgroups.
     `slopes` (fp32, per head): slope * distance is taken off every scaled
-    score."""
+    score. `softcap` > 0: scaled scores pass softcap * tanh(s / softcap)."""
     k = _paged_backend(q)
     if k is not None:
         if tiles is None:
@@ -708,11 +712,50 @@ def paged_attention(out, q, k_cache, v_cache, block_tables, row_seq, positions,
                                 max(1024 // nt, min(4, 2048 // nt))))
         k.paged_attention(out, q, k_cache, v_cache, block_tables, tiles,
                           positions, scale, maps, window, keep_first, sinks,
-                          exact, nsplit, slopes)
+                          exact, nsplit, slopes, softcap)
     else:
         torch_ref.paged_attention(out, q, k_cache, v_cache, block_tables,
                                   row_seq, positions, scale, maps, window,
-                                  keep_first, sinks, slopes)
+                                  keep_first, sinks, slopes, softcap)
+
+
+def head_rope_store(q_out, src, col_q: int, q_heads: int, q_dim: int, q_w,
+                    q_norm_dims: int, q_rot0: int, col_k: int, k_heads: int,
+                    k_dim: int, k_w, k_norm_dims: int, k_rot0: int, col_v: int,
+                    inv_freq, half_layout: bool, amplitude: float, pos32,
+                    k_cache, v_cache, slots, eps: float,
+                    page_groups=None) -> None:
+    """Per-head norm + rotation + cache write (torch_ref.head_rope_store
+    has the semantics). `page_groups` (build_page_groups; GPU, prompts,
+    values read from src): the value rows are written page by page."""
+    k = _paged_backend(src)
+    if k is not None:
+        k.head_rope_store(q_out, src, col_q, q_heads, q_dim, q_w, q_norm_dims,
+                          q_rot0, col_k, k_heads, k_dim, k_w, k_norm_dims,
+                          k_rot0, col_v, inv_freq, half_layout, amplitude,
+                          pos32, k_cache, v_cache, slots, eps, page_groups)
+    else:
+        torch_ref.head_rope_store(q_out, src, col_q, q_heads, q_dim, q_w,
+                                  q_norm_dims, q_rot0, col_k, k_heads, k_dim,
+                                  k_w, k_norm_dims, k_rot0, col_v, inv_freq,
+                                  half_layout, amplitude, pos32, k_cache,
+                                  v_cache, slots, eps)
+
+
+def dual_rms_mix(out, a, wa, b, wb, eps: float) -> None:
+    k = _paged_backend(a)
+    if k is not None:
+        k.dual_rms_mix(out, a, wa, b, wb, eps)
+    else:
+        torch_ref.dual_rms_mix(out, a, wa, b, wb, eps)
+
+
+def head_gate(out, o_hts, gate_src, col: int) -> None:
+    k = _paged_backend(o_hts)
+    if k is not None:
+        k.head_gate(out, o_hts, gate_src, col)
+    else:
+        torch_ref.head_gate(out, o_hts, gate_src, col)
 
 
 def diff_combine(out, a, lam, diff: float, eps: float) -> None:
@@ -826,10 +869,12 @@ def state_scan(y, src, col_x: int, col_b: int, col_c: int, dt_src,
 
 
 def gated_group_norm(out, y, gate, w, groups: int, eps: float,
-                     gate_first: bool) -> None:
+                     gate_first) -> None:
+    """gate_first: True / 1 = silu gate, then norm; False / 0 = norm, then
+    sigmoid gate; 2 = norm, then silu gate."""
     k = _state_backend(y)
     if k is not None:
-        k.gated_group_norm(out, y, gate, w, groups, eps, gate_first)
+        k.gated_group_norm(out, y, gate, w, groups, eps, int(gate_first))
     else:
         torch_ref.gated_group_norm(out, y, gate, w, groups, eps, gate_first)
 
@@ -844,3 +889,21 @@ def route_topk(experts, weights, logits, correction, n_experts: int,
     else:
         torch_ref.route_topk(experts, weights, logits, correction, n_experts,
                              groups, keep, group_top, sigmoid, renorm, scale)
+
+
+def delta_scan(y, src, col_q: int, col_k: int, col_v: int, gate_src,
+               col_a: int, col_b: int, heads: int, groups: int, n_state: int,
+               vdim: int, dt_bias, a_log, state, seq_first, seq_rows,
+               state_slots, pos32, single: bool = False) -> None:
+    """Gated delta rule over the state pool (torch_ref.delta_scan has the
+    semantics). `single`: every sequence brings one row (a decode step)."""
+    k = _state_backend(src)
+    if k is not None:
+        k.delta_scan(y, src, col_q, col_k, col_v, gate_src, col_a, col_b,
+                     heads, groups, n_state, vdim, dt_bias, a_log, state,
+                     seq_first, seq_rows, state_slots, pos32, single)
+    else:
+        torch_ref.delta_scan(y, src, col_q, col_k, col_v, gate_src, col_a,
+                             col_b, heads, groups, n_state, vdim, dt_bias,
+                             a_log, state, seq_first, seq_rows, state_slots,
+                             pos32)

@@ -472,19 +472,23 @@ def sandwich_add_norm(x: torch.Tensor, a: torch.Tensor | None,
                       post_w: torch.Tensor | None, mult: float, eps: float,
                       extra: torch.Tensor | None,
                       next_w: torch.Tensor | None,
-                      h: torch.Tensor | None) -> None:
+                      h: torch.Tensor | None, center: bool = False) -> None:
     """x += mult * rmsnorm(a) * post_w  (+ extra), in fp32 on the fp32
     stream x; then h = rmsnorm(x) * next_w in h's dtype. Either half may be
-    absent (a is None: no sublayer output; next_w is None: no next norm)."""
+    absent (a is None: no sublayer output; next_w is None: no next norm).
+    `center`: both norms take the row's mean off first (weight-only layer
+    norms: deviations over the root of their mean square + eps)."""
+    def unit(t):
+        if center:
+            t = t - t.mean(-1, keepdim=True)
+        return t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps)
+
     if a is not None:
-        af = a.float()
-        y = af * torch.rsqrt(af.pow(2).mean(-1, keepdim=True) + eps)
-        x.add_(y * post_w.float() * mult)
+        x.add_(unit(a.float()) * post_w.float() * mult)
     if extra is not None:
         x.add_(extra.float())
     if next_w is not None:
-        y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
-        h.copy_((y * next_w.float()).to(h.dtype))
+        h.copy_((unit(x) * next_w.float()).to(h.dtype))
 
 
 def rotary_norm_store(q_out: torch.Tensor, qkv: torch.Tensor, nq: int,
@@ -537,7 +541,8 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
                     scale: float, maps: int = 1, window: int = 0,
                     keep_first: int = 0,
                     sinks: torch.Tensor | None = None,
-                    slopes: torch.Tensor | None = None) -> None:
+                    slopes: torch.Tensor | None = None,
+                    softcap: float = 0.0) -> None:
     """out[t, a] = softmax_j(scale * q[t, a] . k_j) . V over the visible
     keys j of row t's sequence: j <= pos(t), and with window > 0 also
     (pos(t) - j < window or j < keep_first). q: [T, A, D] with A = heads *
@@ -545,7 +550,8 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
     [m*D, (m+1)*D) of its kv head's key row and all maps weight the same
     values. sinks (per head, or None) add exp(sink) to the denominator;
     slopes (per head, or None) take slope * (pos(t) - j) off the scaled
-    score."""
+    score; softcap > 0 turns a scaled score s into softcap * tanh(s /
+    softcap) first."""
     T, A, D = q.shape
     nb, G, BS, KW = k_cache.shape
     VW = v_cache.shape[2]
@@ -564,6 +570,8 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
             g = (a // maps) // rep
             m = a % maps
             s = (K[:, g, m * D:(m + 1) * D] @ q[t, a].float()) * scale
+            if softcap:
+                s = softcap * torch.tanh(s / softcap)
             if slopes is not None:
                 s = s - slopes[a // maps].float() * (p - j).float()
             mx = s.max()
@@ -746,18 +754,22 @@ def state_scan(y: torch.Tensor, src: torch.Tensor, col_x: int, col_b: int,
 
 def gated_group_norm(out: torch.Tensor, y: torch.Tensor, gate: torch.Tensor,
                      w: torch.Tensor, groups: int, eps: float,
-                     gate_first: bool) -> None:
-    """gate_first: u = y * silu(gate), then RMS norm of each of `groups`
-    equal parts of the row by its own root mean square, times w. Otherwise:
-    RMS norm of y in parts, times w, times sigmoid(gate). y fp32 [T, C]."""
+                     gate_first) -> None:
+    """gate_first True (1): u = y * silu(gate), then RMS norm of each of
+    `groups` equal parts of the row by its own root mean square, times w.
+    False (0): RMS norm of y in parts, times w, times sigmoid(gate). 2: the
+    same with silu(gate) in place of the sigmoid. y fp32 [T, C]."""
     T, C = y.shape
+    mode = int(gate_first)
     g = gate.float()
-    u = y * (g * torch.sigmoid(g)) if gate_first else y
+    u = y * (g * torch.sigmoid(g)) if mode == 1 else y
     u = u.view(T, groups, C // groups)
     u = (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps)).view(T, C)
     u = u * w.float()
-    if not gate_first:
+    if mode == 0:
         u = u * torch.sigmoid(g)
+    elif mode == 2:
+        u = u * (g * torch.sigmoid(g))
     out.copy_(u.to(out.dtype))
 
 
@@ -789,3 +801,136 @@ def route_topk(experts: torch.Tensor, weights: torch.Tensor,
         wt = wt / (wt.sum(-1, keepdim=True) + 1e-20)
     experts.copy_(idx.to(experts.dtype))
     weights.copy_(wt * scale)
+
+
+# --- rotary row kernel with per-head norms, gated delta rule, row mixes -----
+# (ops/csrc/roperows32.hip, delta_scan.hip)
+
+def head_rope_store(q_out: torch.Tensor | None, src: torch.Tensor, col_q: int,
+                    q_heads: int, q_dim: int, q_w: torch.Tensor | None,
+                    q_norm_dims: int, q_rot0: int, col_k: int, k_heads: int,
+                    k_dim: int, k_w: torch.Tensor | None, k_norm_dims: int,
+                    k_rot0: int, col_v: int, inv_freq: torch.Tensor,
+                    half_layout: bool, amplitude: float, pos32: torch.Tensor,
+                    k_cache: torch.Tensor | None,
+                    v_cache: torch.Tensor | None,
+                    slots: torch.Tensor | None, eps: float) -> None:
+    """Row kernel between a projection and attention. The q side: q_heads
+    heads of q_dim channels at src[:, col_q:]; the k side: k_heads heads of
+    k_dim channels at src[:, col_k:] (k_heads 0: none). Per head, in fp32:
+    the first *_norm_dims channels are RMS-normed over themselves and
+    multiplied by *_w (None: no norm); then the 2 * len(inv_freq) channels
+    from *_rot0 on turn by pos * f (rot0 < 0: no rotation) — channel i with
+    i + half (half_layout) or 2i with 2i+1 — with cos and sin multiplied by
+    `amplitude`. q heads go to q_out [T, q_heads * q_dim]; k heads to their
+    slot of k_cache [nb, G, BS, k_dim]; values to the transposed pages
+    v_cache [nb, G, VW, BS]: src[:, col_v:] (G heads of VW channels), or,
+    with col_v < 0, the first VW channels of each finished key head."""
+    T = src.shape[0]
+    half = inv_freq.numel()
+    ang = pos32.to(torch.float32)[:, None] * inv_freq.float()[None, :]
+    c = (torch.cos(ang) * amplitude)[:, None, :]
+    sn = (torch.sin(ang) * amplitude)[:, None, :]
+
+    def prep(col, heads, dim, w, nd, rot0):
+        t = src[:, col:col + heads * dim].float().reshape(T, heads, dim).clone()
+        if w is not None:
+            part = t[..., :nd]
+            t[..., :nd] = part * torch.rsqrt(
+                part.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+        if rot0 >= 0 and half:
+            r = t[..., rot0:rot0 + 2 * half]
+            if half_layout:
+                u, v = r[..., :half].clone(), r[..., half:].clone()
+                r[..., :half] = u * c - v * sn
+                r[..., half:] = v * c + u * sn
+            else:
+                u, v = r[..., 0::2].clone(), r[..., 1::2].clone()
+                r[..., 0::2] = u * c - v * sn
+                r[..., 1::2] = v * c + u * sn
+        return t
+
+    if q_out is not None and q_heads:
+        q = prep(col_q, q_heads, q_dim, q_w, q_norm_dims, q_rot0)
+        q_out.copy_(q.reshape(T, q_heads * q_dim).to(q_out.dtype))
+    if k_heads and k_cache is not None:
+        nb, G, BS, KW = k_cache.shape
+        VW = v_cache.shape[2]
+        k = prep(col_k, k_heads, k_dim, k_w, k_norm_dims, k_rot0)
+        k = k.to(k_cache.dtype)
+        if col_v >= 0:
+            v = src[:, col_v:col_v + G * VW].reshape(T, G, VW).to(v_cache.dtype)
+        else:
+            v = k[..., :VW]
+        ok = slots >= 0
+        blk, off = slots[ok] // BS, slots[ok] % BS
+        k_cache[blk, :, off] = k[ok]
+        v_cache[blk, :, :, off] = v[ok]
+
+
+def delta_scan(y: torch.Tensor, src: torch.Tensor, col_q: int, col_k: int,
+               col_v: int, gate_src: torch.Tensor, col_a: int, col_b: int,
+               heads: int, groups: int, n_state: int, vdim: int,
+               dt_bias: torch.Tensor, a_log: torch.Tensor,
+               state: torch.Tensor, seq_first: torch.Tensor,
+               seq_rows: torch.Tensor, state_slots: torch.Tensor,
+               pos32: torch.Tensor) -> None:
+    """Gated delta rule, per sequence and head over this step's rows in
+    order, all in fp32:
+        S <- g_t S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;
+        y_t = S^T q_t
+    S [n_state, vdim] is read from state[slot] (zero when the first row
+    sits at position 0) and written back. q = src[:, col_q + g * n_state
+    ...] and k likewise (g = h // (heads / groups)), each scaled to unit
+    length, x / sqrt(sum x^2 + 1e-6), q also by n_state^(-1/2); v =
+    src[:, col_v + h * vdim ...]; g_t = exp(-exp(a_log[h]) *
+    softplus(gate_src[t, col_a + h] + dt_bias[h])), beta_t =
+    sigmoid(gate_src[t, col_b + h]). y: [T, heads * vdim] fp32."""
+    rep = heads // groups
+    for s in range(seq_first.numel()):
+        r0, n, slot = int(seq_first[s]), int(seq_rows[s]), int(state_slots[s])
+        hist = int(pos32[r0])
+        rows = src[r0:r0 + n].float()
+        q = rows[:, col_q:col_q + groups * n_state].view(n, groups, n_state)
+        k = rows[:, col_k:col_k + groups * n_state].view(n, groups, n_state)
+        v = rows[:, col_v:col_v + heads * vdim].view(n, heads, vdim)
+        q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6) \
+            * float(n_state) ** -0.5
+        k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
+        q = q.repeat_interleave(rep, 1)
+        k = k.repeat_interleave(rep, 1)
+        gs = gate_src[r0:r0 + n].float()
+        raw = gs[:, col_a:col_a + heads] + dt_bias.float()
+        dt = raw.clamp(min=0) + torch.log1p(torch.exp(-raw.abs()))
+        g = torch.exp(-torch.exp(a_log.float()) * dt)          # [n, H]
+        beta = torch.sigmoid(gs[:, col_b:col_b + heads])
+        S = (state[slot].clone() if hist > 0
+             else torch.zeros_like(state[slot]))
+        for t in range(n):
+            S = g[t][:, None, None] * S
+            u = beta[t][:, None] * (v[t] - torch.einsum("hnp,hn->hp", S, k[t]))
+            S = S + k[t][:, :, None] * u[:, None, :]
+            y[r0 + t] = torch.einsum("hnp,hn->hp", S, q[t]).reshape(-1)
+        state[slot] = S
+
+
+def dual_rms_mix(out: torch.Tensor, a: torch.Tensor, wa: torch.Tensor,
+                 b: torch.Tensor, wb: torch.Tensor, eps: float) -> None:
+    """out = (rmsnorm(a) * wa + rmsnorm(b) * wb) / 2 over the rows, fp32
+    inside."""
+    def unit(t):
+        t = t.float()
+        return t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps)
+
+    out.copy_((0.5 * (unit(a) * wa.float() + unit(b) * wb.float()))
+              .to(out.dtype))
+
+
+def head_gate(out: torch.Tensor, o_hts: torch.Tensor, gate_src: torch.Tensor,
+              col: int) -> None:
+    """out[t, h * VD + c] = o_hts[h, t, c] * sigmoid(gate_src[t, col + h]):
+    head-major mixer outputs become rows, each head times its gate."""
+    H, T, VD = o_hts.shape
+    g = torch.sigmoid(gate_src[:, col:col + H].float())          # [T, H]
+    o = o_hts.float().transpose(0, 1) * g[:, :, None]
+    out.copy_(o.reshape(T, H * VD).to(out.dtype))
