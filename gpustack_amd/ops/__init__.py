@@ -520,7 +520,8 @@ def latent_attention(ctx, q_lat, cache, block_tables, row_seq, positions,
 
 
 def act_inplace(x, mode: str) -> None:
-    k = _lat_backend(x)
+    # the kernel ships in both fp32-stream libraries: whichever is loaded
+    k = _PAGED if (_PAGED is not None and x.is_cuda) else _lat_backend(x)
     if k is not None:
         k.act_inplace(x, ACT_MODES[mode])
     else:

@@ -30,14 +30,14 @@ LATENT_SOURCES = ["resid32.hip", "latent_attn.hip", "grouped_ff.hip",
 # pre/post-norm fp32-stream row kernels + paged rotary attention (argmax
 # comes with resid32.hip): again a library of its own
 PAGED_SO_PATH = PKG_DIR / "_hip_paged.so"
-PAGED_SOURCES = ["rowmix32.hip", "ragged_attn.hip", "resid32.hip",
-                 "paged_bindings.cpp"]
+PAGED_SOURCES = ["rowmix32.hip", "roperows32.hip", "ragged_attn.hip",
+                 "resid32.hip", "paged_bindings.cpp"]
 
 # layer-norm fp32-stream row kernels, head-norm cache write, scored routing
 # and the recurrent mixers (page-wise value stores come with rowmix32.hip)
 STATE_SO_PATH = PKG_DIR / "_hip_state.so"
-STATE_SOURCES = ["lnrows32.hip", "state_scan.hip", "rowmix32.hip",
-                 "state_bindings.cpp"]
+STATE_SOURCES = ["lnrows32.hip", "state_scan.hip", "delta_scan.hip",
+                 "rowmix32.hip", "state_bindings.cpp"]
 
 
 def _torch_paths():

@@ -10,7 +10,8 @@
 // head are the two halves of differential attention, combined afterwards.
 // A per-head sink logit may join the denominator (no key, no value), and a
 // per-head slope times the distance pos(t) - j may be taken off the scaled
-// score (positions without rotation).
+// score (positions without rotation); a tanh cap may bound the scaled
+// score. q and out are [T, A, *] views with a contiguous last axis.
 //
 // Pools: keys [nblocks, G, BS, KW] with KW = maps * D (rotated at write
 // time), values with every page transposed, [nblocks, G, VW, BS], so both
@@ -62,6 +63,9 @@ struct AttnArgs {
   const float* sinks;        // [A / maps] or null
   const float* slopes;       // [A / maps] or null
   float scale;
+  float softcap;             // > 0: scaled scores pass cap * tanh(s / cap)
+  long q_st, q_sa;           // element strides of q [T, A, D]: row, score map
+  long o_st, o_sa;           // and of out [T, A, VW]
   int T, A, D, VW, KW, G, BS, maps, rep;   // rep = heads / kv heads
   int nseq, maxb, nblocks, window, keep_first;
 };
@@ -100,6 +104,11 @@ DEVICE_INLINE bool key_visible(int j, int pos, int window, int keep_first) {
   return j <= pos && (window <= 0 || pos - j < window || j < keep_first);
 }
 
+DEVICE_INLINE float scaled_score(float dot, const AttnArgs& p) {
+  const float s = dot * p.scale;
+  return p.softcap > 0.f ? p.softcap * tanhf(s / p.softcap) : s;
+}
+
 // ---- exact path ----------------------------------------------------------
 
 template <typename TQ, typename TC, typename TO, int NJ, int KT>
@@ -131,7 +140,7 @@ __global__ __launch_bounds__(THREADS) void paged_attn_exact_kernel(
   const int lo = p.window > 0 ? max(0, jmin - p.window + 1) : 0;
   for (int e = wave; e < G16; e += 4) {
     const bool ok = e < n_ent;
-    const TQ* qp = q + ((long)e_row[e] * p.A + e_a[e]) * D;
+    const TQ* qp = q + (long)e_row[e] * p.q_st + (long)e_a[e] * p.q_sa;
     for (int r = lane; r < D; r += 64) qs[e * D + r] = ok ? ldf(qp + r) : 0.f;
   }
   const int e_s = tid >> 4, kk = tid & 15;
@@ -192,7 +201,8 @@ __global__ __launch_bounds__(THREADS) void paged_attn_exact_kernel(
     for (int u = 0; u < KT / 16; ++u) {
       const int j = k0 + kk + 16 * u;
       s[u] = key_visible(j, my_pos, p.window, p.keep_first)
-                 ? s[u] * p.scale - slope * (float)(my_pos - j) : -INFINITY;
+                 ? scaled_score(s[u], p) - slope * (float)(my_pos - j)
+                 : -INFINITY;
       mx = fmaxf(mx, s[u]);
     }
 #pragma unroll
@@ -245,7 +255,7 @@ __global__ __launch_bounds__(THREADS) void paged_attn_exact_kernel(
     if (e >= n_ent) continue;
     const float l = lsum[e];
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    TO* op = out + ((long)e_row[e] * p.A + e_a[e]) * VW;
+    TO* op = out + (long)e_row[e] * p.o_st + (long)e_a[e] * p.o_sa;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       const int c = lane + 64 * j;
@@ -300,7 +310,8 @@ __global__ __launch_bounds__(THREADS) void paged_attn_mfma_kernel(
   const int lo = p.window > 0 ? max(0, jmin - p.window + 1) : 0;
   for (int e = wave; e < G16; e += 4) {
     const bool ok = e < n_ent;
-    const unsigned short* qp = q + ((long)e_row[e] * p.A + e_a[e]) * D;
+    const unsigned short* qp =
+        q + (long)e_row[e] * p.q_st + (long)e_a[e] * p.q_sa;
     for (int r = lane; r < D; r += 64)
       Ql[e * QS + r] = ok ? qp[r] : (unsigned short)0;
   }
@@ -354,7 +365,7 @@ __global__ __launch_bounds__(THREADS) void paged_attn_mfma_kernel(
       for (int u = 0; u < 4; ++u) {
         const int j = k0 + kk + 16 * u;
         sv[u] = key_visible(j, my_pos, p.window, p.keep_first)
-                    ? Ss[e_s * MSS + kk + 16 * u] * p.scale -
+                    ? scaled_score(Ss[e_s * MSS + kk + 16 * u], p) -
                           slope * (float)(my_pos - j)
                     : -INFINITY;
         mx = fmaxf(mx, sv[u]);
@@ -437,7 +448,7 @@ __global__ __launch_bounds__(THREADS) void paged_attn_mfma_kernel(
     if (e >= n_ent) continue;
     const float l = lsum[e];
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    TO* op = out + ((long)e_row[e] * p.A + e_a[e]) * VW;
+    TO* op = out + (long)e_row[e] * p.o_st + (long)e_a[e] * p.o_sa;
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
       const int ch = (wave + 4 * i) * 16 + lc;
@@ -476,7 +487,7 @@ __global__ __launch_bounds__(MERGE_THREADS) void paged_attn_merge_kernel(
   }
   const float inv = L > 0.f ? 1.0f / L : 0.f;
   const int row = row0 + e / n_a, a = a0 + (e % n_a) * a_step;
-  TO* op = out + ((long)row * p.A + a) * VW;
+  TO* op = out + (long)row * p.o_st + (long)a * p.o_sa;
   for (int ch = threadIdx.x; ch < VW; ch += MERGE_THREADS) {
     float v = 0.f;
     for (int s = 0; s < nsplit; ++s) {
@@ -563,7 +574,8 @@ void paged_attention_launch(void* out, const void* q, const void* k_cache,
                             const void* v_cache, const int* block_tables,
                             const int* tiles, const int* pos32,
                             const float* sinks, const float* slopes,
-                            float scale, int ntiles, int T,
+                            float scale, float softcap, long q_st, long q_sa,
+                            long o_st, long o_sa, int ntiles, int T,
                             int A, int D, int VW, int KW, int G, int BS,
                             int maps, int rep, int nseq, int maxb, int nblocks,
                             int window, int keep_first, int q_bf, int out_bf,
@@ -572,6 +584,8 @@ void paged_attention_launch(void* out, const void* q, const void* k_cache,
   if (ntiles == 0) return;
   AttnArgs p;
   p.block_tables = block_tables; p.tiles = tiles; p.pos32 = pos32;
+  p.softcap = softcap; p.q_st = q_st; p.q_sa = q_sa; p.o_st = o_st;
+  p.o_sa = o_sa;
   p.sinks = sinks; p.slopes = slopes; p.scale = scale; p.T = T; p.A = A; p.D = D; p.VW = VW;
   p.KW = KW; p.G = G; p.BS = BS; p.maps = maps; p.rep = rep; p.nseq = nseq;
   p.maxb = maxb; p.nblocks = nblocks; p.window = window;

@@ -1,0 +1,266 @@
+// Row kernels around attention mixers whose heads are normed and rotated
+// one by one (gfx950).
+//
+//   head_rope_store : per head of a q side and a k side of one projection
+//                     row: RMS norm of the head's first channels with a
+//                     weight vector shared by the heads, then rotation of a
+//                     channel range (pairs (i, i + half) or (2i, 2i + 1),
+//                     cos / sin times an amplitude); q heads out, k heads
+//                     into their page rows, values into the transposed
+//                     value pages — from the projection, or the first
+//                     channels of the finished key head (a latent that is
+//                     key and value at once)
+//   dual_rms_mix    : (rmsnorm(a) * wa + rmsnorm(b) * wb) / 2 per row
+//   head_gate       : head-major outputs -> rows, each head times the
+//                     sigmoid of its gate logit
+//
+// Sums of squares, angles, rotations and gates are fp32 whatever the GEMM
+// dtype; every kernel emits its operand in that dtype directly.
+#include "common.h"
+
+namespace {
+
+template <typename T> DEVICE_INLINE float ld(const T* p);
+template <> DEVICE_INLINE float ld<float>(const float* p) { return *p; }
+template <> DEVICE_INLINE float ld<unsigned short>(const unsigned short* p) {
+  return bf2f(*p);
+}
+template <typename T> DEVICE_INLINE void st(T* p, float v);
+template <> DEVICE_INLINE void st<float>(float* p, float v) { *p = v; }
+template <> DEVICE_INLINE void st<unsigned short>(unsigned short* p, float v) {
+  *p = f2bf(v);
+}
+constexpr int ROW_THREADS = 256;
+
+struct RopeArgs {
+  long ld_src;
+  int col_q, q_heads, q_dim, q_nd, q_rot0;
+  int col_k, k_heads, k_dim, k_nd, k_rot0;
+  int col_v;                 // < 0: values are the key heads' first VW channels
+  const float* q_w;          // [q_nd] or null
+  const float* k_w;          // [k_nd] or null
+  const float* inv_freq;     // [half]
+  int half, half_layout;
+  float amp, eps;
+  const int* pos32;
+  const long* slots;
+  long nslots;
+  int BS, VW, skip_v, T;
+};
+
+// grid (T, ceil((q_heads + k_heads) / 4)): one wave per (row, head). The
+// sin / cos table of the row is built once per workgroup in LDS.
+template <typename TS>
+__global__ __launch_bounds__(ROW_THREADS) void head_rope_store_kernel(
+    TS* __restrict__ q_out, const TS* __restrict__ src,
+    TS* __restrict__ k_cache, TS* __restrict__ v_cache, RopeArgs p) {
+  extern __shared__ float cs_tab[];            // [half] cos, [half] sin
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int half = p.half;
+  const float pos = (float)p.pos32[t];
+  for (int i = threadIdx.x; i < half; i += ROW_THREADS) {
+    float sn, cs;
+    sincosf(pos * p.inv_freq[i], &sn, &cs);
+    cs_tab[i] = cs * p.amp;
+    cs_tab[half + i] = sn * p.amp;
+  }
+  __syncthreads();
+  const int unit = blockIdx.y * 4 + wave;
+  if (unit >= p.q_heads + p.k_heads) return;
+  const bool is_k = unit >= p.q_heads;
+  const int hd = is_k ? unit - p.q_heads : unit;
+  const int dim = is_k ? p.k_dim : p.q_dim;
+  const int nd = is_k ? p.k_nd : p.q_nd;
+  const int rot0 = is_k ? p.k_rot0 : p.q_rot0;
+  const float* w = is_k ? p.k_w : p.q_w;
+  const TS* row = src + (long)t * p.ld_src + (is_k ? p.col_k : p.col_q) +
+                  (long)hd * dim;
+  float inv = 1.f;
+  if (w != nullptr) {
+    float ss = 0.f;
+    for (int c = lane; c < nd; c += 64) {
+      const float v = ld(row + c);
+      ss += v * v;
+    }
+    ss = wave_reduce_sum(ss);
+    inv = 1.0f / sqrtf(ss / (float)nd + p.eps);
+  }
+  long blk = 0;
+  int off = 0;
+  bool store = false;
+  if (is_k) {
+    const long slot = p.slots[t];
+    store = slot >= 0 && slot < p.nslots;
+    if (!store) return;
+    blk = slot / p.BS;
+    off = (int)(slot % p.BS);
+  }
+  const int G = p.k_heads;
+  for (int c = lane; c < dim; c += 64) {
+    float v = ld(row + c);
+    if (w != nullptr && c < nd) v = v * inv * w[c];
+    const int r = c - rot0;
+    if (rot0 >= 0 && r >= 0 && r < 2 * half) {
+      int i, pc;
+      bool lower;
+      if (p.half_layout) {
+        lower = r < half;
+        i = lower ? r : r - half;
+        pc = lower ? c + half : c - half;
+      } else {
+        lower = (r & 1) == 0;
+        i = r >> 1;
+        pc = lower ? c + 1 : c - 1;
+      }
+      float o = ld(row + pc);
+      if (w != nullptr && pc < nd) o = o * inv * w[pc];
+      const float cs = cs_tab[i], sn = cs_tab[half + i];
+      v = lower ? v * cs - o * sn : v * cs + o * sn;
+    }
+    if (!is_k) {
+      st(q_out + ((long)t * p.q_heads + hd) * dim + c, v);
+    } else {
+      st(k_cache + ((blk * G + hd) * p.BS + off) * (long)dim + c, v);
+      if (p.col_v < 0 && c < p.VW)
+        st(v_cache + ((blk * G + hd) * (long)p.VW + c) * p.BS + off, v);
+    }
+  }
+  if (is_k && p.col_v >= 0 && !p.skip_v) {
+    const TS* vs = src + (long)t * p.ld_src + p.col_v + (long)hd * p.VW;
+    for (int c = lane; c < p.VW; c += 64)
+      v_cache[((blk * G + hd) * (long)p.VW + c) * p.BS + off] = vs[c];
+  }
+}
+
+DEVICE_INLINE float block_sum(float v, float* red) {
+  v = wave_reduce_sum(v);
+  const int w = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  return red[0] + red[1] + red[2] + red[3];
+}
+
+// One workgroup per row; NV values of each input stay in registers between
+// the sums of squares and the store (W <= NV * 256), wider rows re-read.
+template <typename TS, int NV>
+__global__ __launch_bounds__(ROW_THREADS) void dual_rms_mix_kernel(
+    TS* __restrict__ out, const TS* __restrict__ a, const float* __restrict__ wa,
+    const TS* __restrict__ b, const float* __restrict__ wb, int W, float eps) {
+  __shared__ float red[4];
+  const long t = blockIdx.x;
+  const TS* ar = a + t * W;
+  const TS* br = b + t * W;
+  float ka[NV], kb[NV];
+  float sa = 0.f, sb = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int i = threadIdx.x + j * ROW_THREADS;
+    ka[j] = i < W ? ld(ar + i) : 0.f;
+    kb[j] = i < W ? ld(br + i) : 0.f;
+    sa += ka[j] * ka[j];
+    sb += kb[j] * kb[j];
+  }
+  for (int i = threadIdx.x + NV * ROW_THREADS; i < W; i += ROW_THREADS) {
+    const float x = ld(ar + i), y = ld(br + i);
+    sa += x * x;
+    sb += y * y;
+  }
+  sa = block_sum(sa, red);
+  sb = block_sum(sb, red);
+  const float ia = 1.0f / sqrtf(sa / (float)W + eps);
+  const float ib = 1.0f / sqrtf(sb / (float)W + eps);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int i = threadIdx.x + j * ROW_THREADS;
+    if (i < W)
+      st(out + t * W + i, 0.5f * (ka[j] * ia * wa[i] + kb[j] * ib * wb[i]));
+  }
+  for (int i = threadIdx.x + NV * ROW_THREADS; i < W; i += ROW_THREADS)
+    st(out + t * W + i,
+       0.5f * (ld(ar + i) * ia * wa[i] + ld(br + i) * ib * wb[i]));
+}
+
+template <typename TS>
+__global__ __launch_bounds__(256) void head_gate_kernel(
+    TS* __restrict__ out, const TS* __restrict__ o_hts,
+    const TS* __restrict__ gate_src, long ld_gate, int col, int H, int T,
+    int VD) {
+  const long n = (long)T * H * VD;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long)gridDim.x * blockDim.x) {
+    const int c = (int)(i % VD);
+    const long th = i / VD;
+    const int h = (int)(th % H);
+    const long t = th / H;
+    const float g = ld(gate_src + t * ld_gate + col + h);
+    const float v = ld(o_hts + ((long)h * T + t) * VD + c);
+    st(out + i, v / (1.0f + expf(-g)));
+  }
+}
+
+}  // namespace
+
+void head_rope_store_launch(void* q_out, const void* src, long ld_src,
+                            int col_q, int q_heads, int q_dim,
+                            const float* q_w, int q_nd, int q_rot0, int col_k,
+                            int k_heads, int k_dim, const float* k_w, int k_nd,
+                            int k_rot0, int col_v, const float* inv_freq,
+                            int half, int half_layout, float amp,
+                            const int* pos32, void* k_cache, void* v_cache,
+                            const long* slots, long nslots, int BS, int VW,
+                            float eps, int skip_v, int T, int bf,
+                            hipStream_t s) {
+  if (T <= 0 || q_heads + k_heads <= 0) return;
+  RopeArgs p;
+  p.ld_src = ld_src; p.col_q = col_q; p.q_heads = q_heads; p.q_dim = q_dim;
+  p.q_nd = q_nd; p.q_rot0 = q_rot0; p.col_k = col_k; p.k_heads = k_heads;
+  p.k_dim = k_dim; p.k_nd = k_nd; p.k_rot0 = k_rot0; p.col_v = col_v;
+  p.q_w = q_w; p.k_w = k_w; p.inv_freq = inv_freq; p.half = half;
+  p.half_layout = half_layout; p.amp = amp; p.eps = eps; p.pos32 = pos32;
+  p.slots = slots; p.nslots = nslots; p.BS = BS; p.VW = VW; p.skip_v = skip_v;
+  p.T = T;
+  const dim3 grid(T, (q_heads + k_heads + 3) / 4);
+  const size_t tab = (size_t)2 * half * sizeof(float);
+  if (bf)
+    head_rope_store_kernel<unsigned short><<<grid, ROW_THREADS, tab, s>>>(
+        (unsigned short*)q_out, (const unsigned short*)src,
+        (unsigned short*)k_cache, (unsigned short*)v_cache, p);
+  else
+    head_rope_store_kernel<float><<<grid, ROW_THREADS, tab, s>>>(
+        (float*)q_out, (const float*)src, (float*)k_cache, (float*)v_cache, p);
+}
+
+void dual_rms_mix_launch(void* out, const void* a, const float* wa,
+                         const void* b, const float* wb, int T, int W,
+                         float eps, int bf, hipStream_t s) {
+  if (T <= 0) return;
+#define DRM(TS, NV)                                                         \
+  dual_rms_mix_kernel<TS, NV><<<T, ROW_THREADS, 0, s>>>(                    \
+      (TS*)out, (const TS*)a, wa, (const TS*)b, wb, W, eps)
+  if (bf) {
+    if (W <= 4 * ROW_THREADS) DRM(unsigned short, 4);
+    else DRM(unsigned short, 16);
+  } else {
+    if (W <= 4 * ROW_THREADS) DRM(float, 4);
+    else DRM(float, 16);
+  }
+#undef DRM
+}
+
+void head_gate_launch(void* out, const void* o_hts, const void* gate_src,
+                      long ld_gate, int col, int H, int T, int VD, int bf,
+                      hipStream_t s) {
+  const long n = (long)T * H * VD;
+  if (n <= 0) return;
+  const int grid = (int)min((n + 255) / 256, (long)(256 * 32));
+  if (bf)
+    head_gate_kernel<unsigned short><<<grid, 256, 0, s>>>(
+        (unsigned short*)out, (const unsigned short*)o_hts,
+        (const unsigned short*)gate_src, ld_gate, col, H, T, VD);
+  else
+    head_gate_kernel<float><<<grid, 256, 0, s>>>(
+        (float*)out, (const float*)o_hts, (const float*)gate_src, ld_gate, col,
+        H, T, VD);
+}

@@ -9,7 +9,8 @@
 //
 //   sandwich_add_norm : x += mult * rmsnorm(a) * post_w (+ extra);
 //                       h = rmsnorm(x) * next_w          (closes one
-//                       sublayer and opens the next in one pass)
+//                       sublayer and opens the next in one pass; RMS norms
+//                       or, centred, weight-only layer norms)
 //   rotary_norm_store : optional whole-row RMS norm of q and k, pairwise
 //                       rotary, q out, k and v into their paged pools
 //   diff_combine      : unit_rms(a1 - lambda * a2) * (1 - diff) per head
@@ -51,59 +52,82 @@ __global__ __launch_bounds__(ROW_THREADS) void embed_rows_kernel(
 }
 
 // NV: row values each lane keeps in registers between the two halves
-// (W <= NV * 256); wider rows re-read x.
+// (W <= NV * 256); wider rows re-read x. center: both norms take the row's
+// mean off first (weight-only layer norms).
 template <typename TA, typename TH, int NV>
 __global__ __launch_bounds__(ROW_THREADS) void sandwich_add_norm_kernel(
     float* __restrict__ x, const TA* __restrict__ a,
     const float* __restrict__ post_w, float mult,
     const float* __restrict__ extra, const float* __restrict__ next_w,
-    TH* __restrict__ h, int W, float eps) {
+    TH* __restrict__ h, int W, float eps, int center) {
   __shared__ float red[4];
   const long t = blockIdx.x;
   float* xr = x + t * W;
-  float inv_a = 0.f;
+  float inv_a = 0.f, mean_a = 0.f;
   if (a != nullptr) {
     const TA* ar = a + t * W;
+    if (center) {
+      float s1 = 0.f;
+      for (int i = threadIdx.x; i < W; i += ROW_THREADS) s1 += ld(ar + i);
+      mean_a = block_sum(s1, red) / (float)W;
+    }
     float ss = 0.f;
     for (int i = threadIdx.x; i < W; i += ROW_THREADS) {
-      const float v = ld(ar + i);
+      const float v = ld(ar + i) - mean_a;
       ss += v * v;
     }
     ss = block_sum(ss, red);
     inv_a = 1.0f / sqrtf(ss / (float)W + eps);
   }
   float keep[NV];
-  float sx = 0.f;
+  float sx = 0.f, s1x = 0.f;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int i = threadIdx.x + j * ROW_THREADS;
     float v = 0.f;
     if (i < W) {
       v = xr[i];
-      if (a != nullptr) v += (ld(a + t * W + i) * inv_a * post_w[i]) * mult;
+      if (a != nullptr)
+        v += ((ld(a + t * W + i) - mean_a) * inv_a * post_w[i]) * mult;
       if (extra != nullptr) v += extra[t * W + i];
       if (a != nullptr || extra != nullptr) xr[i] = v;
     }
     keep[j] = v;
     sx += v * v;
+    s1x += v;
   }
   for (int i = threadIdx.x + NV * ROW_THREADS; i < W; i += ROW_THREADS) {
     float v = xr[i];
-    if (a != nullptr) v += (ld(a + t * W + i) * inv_a * post_w[i]) * mult;
+    if (a != nullptr)
+      v += ((ld(a + t * W + i) - mean_a) * inv_a * post_w[i]) * mult;
     if (extra != nullptr) v += extra[t * W + i];
     if (a != nullptr || extra != nullptr) xr[i] = v;
     sx += v * v;
+    s1x += v;
   }
   if (next_w == nullptr) return;
+  float mean_x = 0.f;
+  if (center) {
+    // the deviations' squares, summed as such (no E[x^2] - mean^2)
+    mean_x = block_sum(s1x, red) / (float)W;
+    sx = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int i = threadIdx.x + j * ROW_THREADS;
+      if (i < W) sx += (keep[j] - mean_x) * (keep[j] - mean_x);
+    }
+    for (int i = threadIdx.x + NV * ROW_THREADS; i < W; i += ROW_THREADS)
+      sx += (xr[i] - mean_x) * (xr[i] - mean_x);
+  }
   sx = block_sum(sx, red);
   const float inv_x = 1.0f / sqrtf(sx / (float)W + eps);
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int i = threadIdx.x + j * ROW_THREADS;
-    if (i < W) st(h + t * W + i, keep[j] * inv_x * next_w[i]);
+    if (i < W) st(h + t * W + i, (keep[j] - mean_x) * inv_x * next_w[i]);
   }
   for (int i = threadIdx.x + NV * ROW_THREADS; i < W; i += ROW_THREADS)
-    st(h + t * W + i, xr[i] * inv_x * next_w[i]);
+    st(h + t * W + i, (xr[i] - mean_x) * inv_x * next_w[i]);
 }
 
 // W % 4 == 0 and W <= NV * 1024: four consecutive channels per lane and
@@ -133,28 +157,40 @@ __global__ __launch_bounds__(ROW_THREADS) void sandwich_add_norm_vec_kernel(
     float* __restrict__ x, const TA* __restrict__ a,
     const float* __restrict__ post_w, float mult,
     const float* __restrict__ extra, const float* __restrict__ next_w,
-    TH* __restrict__ h, int W, float eps) {
+    TH* __restrict__ h, int W, float eps, int center) {
   __shared__ float red[4];
   const long t = blockIdx.x;
   float* xr = x + t * W;
   float av[NV][4];
   float inv_a = 0.f;
   if (a != nullptr) {
-    float ss = 0.f;
+    float s1 = 0.f;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int i = (threadIdx.x + j * ROW_THREADS) * 4;
       if (i < W) {
         Vec4<TA>::load(a + t * W + i, av[j]);
-        ss += av[j][0] * av[j][0] + av[j][1] * av[j][1] +
-              av[j][2] * av[j][2] + av[j][3] * av[j][3];
+        s1 += av[j][0] + av[j][1] + av[j][2] + av[j][3];
+      }
+    }
+    const float mean_a = center ? block_sum(s1, red) / (float)W : 0.f;
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int i = (threadIdx.x + j * ROW_THREADS) * 4;
+      if (i < W) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          av[j][k] -= mean_a;
+          ss += av[j][k] * av[j][k];
+        }
       }
     }
     ss = block_sum(ss, red);
     inv_a = 1.0f / sqrtf(ss / (float)W + eps);
   }
   float keep[NV][4];
-  float sx = 0.f;
+  float sx = 0.f, s1x = 0.f;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int i = (threadIdx.x + j * ROW_THREADS) * 4;
@@ -174,10 +210,27 @@ __global__ __launch_bounds__(ROW_THREADS) void sandwich_add_norm_vec_kernel(
       }
       if (a != nullptr || extra != nullptr) Vec4<float>::store(xr + i, keep[j]);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) sx += keep[j][k] * keep[j][k];
+      for (int k = 0; k < 4; ++k) {
+        sx += keep[j][k] * keep[j][k];
+        s1x += keep[j][k];
+      }
     }
   }
   if (next_w == nullptr) return;
+  float mean_x = 0.f;
+  if (center) {
+    mean_x = block_sum(s1x, red) / (float)W;
+    sx = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int i = (threadIdx.x + j * ROW_THREADS) * 4;
+      if (i < W) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          sx += (keep[j][k] - mean_x) * (keep[j][k] - mean_x);
+      }
+    }
+  }
   sx = block_sum(sx, red);
   const float inv_x = 1.0f / sqrtf(sx / (float)W + eps);
 #pragma unroll
@@ -187,7 +240,7 @@ __global__ __launch_bounds__(ROW_THREADS) void sandwich_add_norm_vec_kernel(
       float w[4], o[4];
       Vec4<float>::load(next_w + i, w);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) o[k] = keep[j][k] * inv_x * w[k];
+      for (int k = 0; k < 4; ++k) o[k] = (keep[j][k] - mean_x) * inv_x * w[k];
       Vec4<TH>::store(h + t * W + i, o);
     }
   }
@@ -552,8 +605,9 @@ void embed_rows_f32_launch(float* x, const long* tokens, const void* embed,
 template <typename TA, typename TH>
 static void sandwich_pick(float* x, const void* a, const float* post_w,
                           float mult, const float* extra, const float* next_w,
-                          void* h, int T, int W, float eps, hipStream_t s) {
-#define SW_ARGS x, (const TA*)a, post_w, mult, extra, next_w, (TH*)h, W, eps
+                          void* h, int T, int W, float eps, int center,
+                          hipStream_t s) {
+#define SW_ARGS x, (const TA*)a, post_w, mult, extra, next_w, (TH*)h, W, eps, center
   if (W % 4 == 0 && W <= 8 * 1024) {
     if (W <= 1024)
       sandwich_add_norm_vec_kernel<TA, TH, 1><<<T, ROW_THREADS, 0, s>>>(SW_ARGS);
@@ -575,16 +629,17 @@ static void sandwich_pick(float* x, const void* a, const float* post_w,
 void sandwich_add_norm_launch(float* x, const void* a, const float* post_w,
                               float mult, const float* extra,
                               const float* next_w, void* h, int T, int W,
-                              float eps, int a_bf, int h_bf, hipStream_t s) {
+                              float eps, int a_bf, int h_bf, int center,
+                              hipStream_t s) {
   if (T <= 0) return;
   if (a_bf && h_bf)
-    sandwich_pick<unsigned short, unsigned short>(x, a, post_w, mult, extra, next_w, h, T, W, eps, s);
+    sandwich_pick<unsigned short, unsigned short>(x, a, post_w, mult, extra, next_w, h, T, W, eps, center, s);
   else if (a_bf)
-    sandwich_pick<unsigned short, float>(x, a, post_w, mult, extra, next_w, h, T, W, eps, s);
+    sandwich_pick<unsigned short, float>(x, a, post_w, mult, extra, next_w, h, T, W, eps, center, s);
   else if (h_bf)
-    sandwich_pick<float, unsigned short>(x, a, post_w, mult, extra, next_w, h, T, W, eps, s);
+    sandwich_pick<float, unsigned short>(x, a, post_w, mult, extra, next_w, h, T, W, eps, center, s);
   else
-    sandwich_pick<float, float>(x, a, post_w, mult, extra, next_w, h, T, W, eps, s);
+    sandwich_pick<float, float>(x, a, post_w, mult, extra, next_w, h, T, W, eps, center, s);
 }
 
 void rotary_norm_store_launch(void* q_out, const void* qkv, long ld_qkv, int nq,

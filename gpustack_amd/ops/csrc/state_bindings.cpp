@@ -1,5 +1,6 @@
 // Torch bindings for the layer-norm row kernels, the head-norm cache write,
-// scored routing (lnrows32.hip) and the recurrent mixers (state_scan.hip);
+// scored routing (lnrows32.hip) and the recurrent mixers (state_scan.hip,
+// delta_scan.hip);
 // page-wise value stores come from rowmix32.hip. Every shape a kernel or its
 // grid assumes is checked here on the host before the launch; VALUES inside
 // index tensors are bounded in the kernels.
@@ -15,6 +16,8 @@ void route_topk_launch(int*, float*, const float*, int, const float*, int, int, 
 void causal_conv_silu_launch(void*, const void*, long, int, int, int, const float*, const float*, void*, const int*, const int*, const int*, const int*, const int*, int, int, int, int, hipStream_t);
 int state_scan_launch(float*, const void*, long, int, int, int, const void*, long, int, int, int, int, int, int, const float*, const float*, const float*, const float*, float*, const int*, const int*, const int*, const int*, int, int, int, int, int, hipStream_t);
 void gated_group_norm_launch(void*, const float*, const void*, long, const float*, int, int, int, float, int, int, int, hipStream_t);
+int delta_scan_launch(float*, const void*, long, int, int, int, const void*, long, int, int, int, int, int, int, const float*, const float*, float*, const int*, const int*, const int*, const int*, int, int, int, int, int, hipStream_t);
+int delta_scan_max_state();
 int state_scan_max_state();
 int conv_max_taps();
 
@@ -296,8 +299,47 @@ void state_scan(Tensor y, Tensor src, long col_x, long col_b, long col_c,
   HIP_CHECK_LAST();
 }
 
+void delta_scan(Tensor y, Tensor src, long col_q, long col_k, long col_v,
+                Tensor gate_src, long col_a, long col_b, long heads,
+                long groups, long n_state, long vdim, Tensor dt_bias,
+                Tensor a_log, Tensor state, Tensor seq_first, Tensor seq_rows,
+                Tensor state_slots, Tensor pos32, bool single) {
+  chk(y, "y", at::kFloat);
+  chk(state, "state", at::kFloat);
+  chk(dt_bias, "dt_bias", at::kFloat);
+  chk(a_log, "a_log", at::kFloat);
+  const int bf = view_kind(src, "src");
+  const int T = src.size(0);
+  TORCH_CHECK(heads >= 1 && groups >= 1 && heads % groups == 0 &&
+              n_state >= 1 && n_state <= delta_scan_max_state() && vdim >= 1);
+  TORCH_CHECK(y.dim() == 2 && y.size(0) == T && y.size(1) == heads * vdim);
+  TORCH_CHECK(state.dim() == 4 && state.size(0) >= 1 && state.size(1) == heads &&
+              state.size(2) == n_state && state.size(3) == vdim,
+              "state must be [slots, heads, state, vdim]");
+  const long W = src.size(1);
+  TORCH_CHECK(col_v >= 0 && col_v + heads * vdim <= W && col_q >= 0 &&
+              col_q + groups * n_state <= W && col_k >= 0 &&
+              col_k + groups * n_state <= W, "columns outside the source");
+  TORCH_CHECK(view_kind(gate_src, "gate_src") == bf && gate_src.size(0) == T &&
+              col_a >= 0 && col_a + heads <= gate_src.size(1) && col_b >= 0 &&
+              col_b + heads <= gate_src.size(1), "gate columns outside");
+  TORCH_CHECK(dt_bias.numel() == heads && a_log.numel() == heads);
+  const int nseq = seq_view(seq_first, seq_rows, state_slots, pos32, T);
+  const int ok = delta_scan_launch(
+      y.data_ptr<float>(), src.data_ptr(), src.stride(0), (int)col_q,
+      (int)col_k, (int)col_v, gate_src.data_ptr(), gate_src.stride(0),
+      (int)col_a, (int)col_b, (int)heads, (int)groups, (int)n_state, (int)vdim,
+      dt_bias.data_ptr<float>(), a_log.data_ptr<float>(),
+      state.data_ptr<float>(), seq_first.data_ptr<int>(),
+      seq_rows.data_ptr<int>(), state_slots.data_ptr<int>(),
+      pos32.data_ptr<int>(), nseq, (int)state.size(0), T, bf, single ? 1 : 0,
+      cur_stream(src));
+  TORCH_CHECK(ok, "state size unsupported");
+  HIP_CHECK_LAST();
+}
+
 void gated_group_norm(Tensor out, Tensor y, Tensor gate, Tensor w, long groups,
-                      double eps, bool gate_first) {
+                      double eps, long gate_first) {
   chk(y, "y", at::kFloat);
   chk(w, "w", at::kFloat);
   const int out_bf = act_kind(out, "out");
@@ -306,9 +348,10 @@ void gated_group_norm(Tensor out, Tensor y, Tensor gate, Tensor w, long groups,
               gate.size(0) == y.size(0) && gate.size(1) == y.size(1));
   const int T = y.size(0), C = y.size(1);
   TORCH_CHECK(groups >= 1 && C % groups == 0 && w.numel() == C);
+  TORCH_CHECK(gate_first >= 0 && gate_first <= 2);
   gated_group_norm_launch(out.data_ptr(), y.data_ptr<float>(), gate.data_ptr(),
                           gate.stride(0), w.data_ptr<float>(), T, C,
-                          (int)groups, (float)eps, gate_first ? 1 : 0, gate_bf,
+                          (int)groups, (float)eps, (int)gate_first, gate_bf,
                           out_bf, cur_stream(y));
   HIP_CHECK_LAST();
 }
@@ -322,5 +365,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("route_topk", &route_topk);
   m.def("causal_conv_silu", &causal_conv_silu);
   m.def("state_scan", &state_scan);
+  m.def("delta_scan", &delta_scan);
   m.def("gated_group_norm", &gated_group_norm);
 }

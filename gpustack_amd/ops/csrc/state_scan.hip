@@ -21,8 +21,8 @@
 //                      decay, step), then walked in order. Step sizes and
 //                      decays are computed here in fp32: a = exp(-exp(A_log)
 //                      * dt), b = dt = softplus(raw + bias), or constants.
-//   gated_group_norm : gate and RMS norm in equal parts of the row, in
-//                      either order
+//   gated_group_norm : gate (SiLU or sigmoid) and RMS norm in equal parts of
+//                      the row, in either order
 #include "common.h"
 
 namespace {
@@ -527,8 +527,9 @@ DEVICE_INLINE float block_sum(float v, float* red) {
   return red[0] + red[1] + red[2] + red[3];
 }
 
-// grid (T, groups): one workgroup per (row, part). gate_first: u = y *
-// silu(gate), out = u / rms(u) * w; else out = y / rms(y) * w * sigmoid(gate).
+// grid (T, groups): one workgroup per (row, part). gate_first 1: u = y *
+// silu(gate), out = u / rms(u) * w; 0: out = y / rms(y) * w * sigmoid(gate);
+// 2: out = y / rms(y) * w * silu(gate).
 template <typename TG, typename TO>
 __global__ __launch_bounds__(ROW_THREADS) void gated_group_norm_kernel(
     TO* __restrict__ out, const float* __restrict__ y,
@@ -542,7 +543,7 @@ __global__ __launch_bounds__(ROW_THREADS) void gated_group_norm_kernel(
   float ss = 0.f;
   for (int i = threadIdx.x; i < gs; i += ROW_THREADS) {
     float u = yr[i];
-    if (gate_first) u *= silu_f(ld(gr + i));
+    if (gate_first == 1) u *= silu_f(ld(gr + i));
     ss += u * u;
   }
   ss = block_sum(ss, red);
@@ -550,7 +551,8 @@ __global__ __launch_bounds__(ROW_THREADS) void gated_group_norm_kernel(
   for (int i = threadIdx.x; i < gs; i += ROW_THREADS) {
     const float gv = ld(gr + i);
     float u = yr[i];
-    if (gate_first) u = u * silu_f(gv) * inv * w[c0 + i];
+    if (gate_first == 1) u = u * silu_f(gv) * inv * w[c0 + i];
+    else if (gate_first == 2) u = u * inv * w[c0 + i] * silu_f(gv);
     else u = u * inv * w[c0 + i] * sigmoid_f(gv);
     st(out + t * C + c0 + i, u);
   }
@@ -580,7 +582,7 @@ __global__ __launch_bounds__(ROW_THREADS) void gated_group_norm_vec_kernel(
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         gv[j][k] = bf2f(g4[k]);
-        u[j][k] = gate_first ? yv[k] * silu_f(gv[j][k]) : yv[k];
+        u[j][k] = gate_first == 1 ? yv[k] * silu_f(gv[j][k]) : yv[k];
         ss += u[j][k] * u[j][k];
       }
     }
@@ -596,7 +598,8 @@ __global__ __launch_bounds__(ROW_THREADS) void gated_group_norm_vec_kernel(
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         float r = u[j][k] * inv * wv[k];
-        if (!gate_first) r *= sigmoid_f(gv[j][k]);
+        if (gate_first == 0) r *= sigmoid_f(gv[j][k]);
+        else if (gate_first == 2) r *= silu_f(gv[j][k]);
         o[k] = f2bf(r);
       }
       *reinterpret_cast<u16x4*>(out + t * C + c0 + i) = o;
