@@ -254,3 +254,156 @@ def forward(cfg, w, tokens, return_layers=False):
     if return_layers:
         return logits, torch.stack(stream)
     return logits
+
+
+def greedy(cfg, w, prompt, n):
+    """n greedy tokens after `prompt`, recomputing the whole sequence."""
+    toks, out = list(prompt), []
+    for _ in range(n):
+        nxt = int(forward(cfg, w, toks)[-1].argmax())
+        out.append(nxt)
+        toks.append(nxt)
+    return out
+
+
+# ---- small configurations and random checkpoints for the tests ----------------
+
+def rot_entry(dims, base=100.0, factor=4.0, original=16, fast=4.0, slow=1.0,
+              scaling=True):
+    r = {"dims": dims, "base": base}
+    if scaling:
+        r["scaling"] = {"factor": factor, "original": original, "fast": fast,
+                        "slow": slow}
+    return r
+
+
+def latent_layer(heads=3, dim=6, rot_dim=4, vdim=5, kv_rank=10, q_rank=7,
+                 window=9, scale=0.4, ff=20, kv_from=None, **rot):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim,
+         "kv_rank": kv_rank, "q_rank": q_rank, "scale": scale,
+         "mask": {"size": window}, "rot": rot_entry(rot_dim, **rot)}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return {"type": "latent_attention", "mixer": m,
+            "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def delta_mixer_entry(heads=4, kv_heads=2, dim=6, vdim=5, conv=3):
+    return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+            "conv": conv}
+
+
+def delta_layer(ff=0, **kw):
+    return {"type": "delta", "mixer": delta_mixer_entry(**kw),
+            "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def softmax_entry(heads=4, kv_heads=2, dim=8, vdim=6, rot_dims=4, scale=0.5,
+                  softcap=3.0, **rot):
+    return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+            "scale": scale, "softcap": softcap,
+            "rot": rot_entry(rot_dims, **rot)}
+
+
+def parallel_layer(left=None, right=None, ff=16):
+    return {"type": "parallel",
+            "mixer": {"left": left or softmax_entry(),
+                      "right": right or delta_mixer_entry(heads=2, kv_heads=1,
+                                                          dim=4, vdim=6,
+                                                          conv=4)},
+            "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def make_config(width=24, vocab=50, layers=None, eps=1e-5):
+    if layers is None:
+        layers = [latent_layer(), delta_layer(), parallel_layer(),
+                  latent_layer(window=5, kv_from=0, ff=12)]
+    return {"architecture": "Makezen", "vocab": vocab, "width": width,
+            "norm": {"eps": eps}, "layers": layers}
+
+
+def make_weights(cfg, seed=0):
+    """Random bf16 checkpoint of a configuration (norm weights, sinks,
+    biases and decay constants spread enough to matter)."""
+    g = torch.Generator().manual_seed(seed)
+    W = cfg["width"]
+    w = {}
+
+    def lin(name, out, inp, gain=1.0):
+        w[name] = (torch.randn(out, inp, generator=g) * gain * inp ** -0.5
+                   ).to(torch.bfloat16)
+
+    def vec(name, n, base=1.0, std=0.2):
+        w[name] = (base + std * torch.randn(n, generator=g)).to(torch.bfloat16)
+
+    def delta(p, m):
+        H, G, N, P = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        for nm, rows in (("q", G * N), ("k", G * N), ("v", H * P)):
+            lin(p + nm, rows, W, 1.5)
+            w[p + nm + ".conv"] = (torch.randn(rows, m["conv"], generator=g)
+                                   * 0.6).to(torch.bfloat16)
+        lin(p + "b", H, W, 2.0)
+        lin(p + "a", H, W, 2.0)
+        lin(p + "g", H * P, W, 1.5)
+        vec(p + "A_log", H, -1.0, 1.0)
+        vec(p + "dt_bias", H, 0.0, 1.0)
+        vec(p + "norm", P)
+        lin(p + "o", W, H * P)
+
+    def softmax(p, m):
+        H, G, D, VD = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        for nm, rows in (("q", H * D), ("k", G * D), ("v", G * VD)):
+            lin(p + nm, rows, W, 1.5)
+            vec(p + nm + ".b", rows, 0.0, 0.3)
+        vec(p + "q.norm", D, 1.0, 0.3)
+        vec(p + "k.norm", D, 1.0, 0.3)
+        lin(p + "o", W, H * VD)
+
+    w["embed"] = torch.randn(cfg["vocab"], W, generator=g).to(torch.bfloat16)
+    vec("embed.norm", W)
+    vec("final.norm", W)
+    for i, ent in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", ent["mixer"]
+        vec(p + "norm1", W)
+        vec(p + "norm1b", W)
+        if ent["type"] == "delta":
+            delta(p + "mix.", m)
+        elif ent["type"] == "parallel":
+            softmax(p + "mix.left.", m["left"])
+            delta(p + "mix.right.", m["right"])
+            vec(p + "mix.left.out", W)
+            vec(p + "mix.right.out", W)
+        else:
+            H, D, RD, VD = m["heads"], m["dim"], m["rot_dim"], m["vdim"]
+            R, QR = m["kv_rank"], m["q_rank"]
+            lin(p + "mix.dq", QR, W)
+            vec(p + "mix.dq.norm", QR)
+            lin(p + "mix.uq", H * (D + RD), QR, 1.5)
+            if m.get("kv_from") is None:
+                lin(p + "mix.dkv", R + RD, W, 1.5)
+                vec(p + "mix.dkv.norm", R)
+            lin(p + "mix.uk", H * D, R, 1.5)
+            lin(p + "mix.uv", H * VD, R, 1.5)
+            vec(p + "mix.sink", H, 0.0, 1.0)
+            lin(p + "mix.g", H, W, 2.0)
+            lin(p + "mix.o", W, H * VD)
+        if ent.get("mlp"):
+            vec(p + "norm2", W)
+            vec(p + "norm2b", W)
+            lin(p + "mlp.up", ent["mlp"]["ff"], W)
+            lin(p + "mlp.down", W, ent["mlp"]["ff"])
+    return w
+
+
+def save_model(path, cfg, weights):
+    import json
+    from pathlib import Path
+
+    from safetensors.torch import save_file
+
+    path = Path(path)
+    path.mkdir(parents=True, exist_ok=True)
+    (path / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.contiguous() for k, v in weights.items()},
+              str(path / "model.safetensors"))
+    return str(path)
