@@ -56,13 +56,13 @@ def parse_args():
                     help="prefill-context-parallel degree (rows chunked "
                          "across ranks, replicated decode); world = tp*cp")
     ap.add_argument("--layer-bench", action="store_true",
-                    help="instead of the serving workload: Vunitar or Fusipel "
-                         "layers (--layer-family) at "
-                         "real-model sizes beside the closest llama-lineage "
+                    help="instead of the serving workload: Vunitar, Fusipel, "
+                         "Livasun or Makezen layers (--layer-family) at "
+                         "real-model sizes beside the closest existing "
                          "stack (prefill/decode tok/s + per-kernel roofline "
                          "shares; gpustack_amd/bench/layer_bench.py)")
     ap.add_argument("--layer-family", default="vunitar",
-                    choices=["vunitar", "fusipel", "livasun"],
+                    choices=["vunitar", "fusipel", "livasun", "makezen"],
                     help="model family measured by --layer-bench")
     ap.add_argument("--layer-sizes", default="small,medium",
                     help="comma list of small,medium,large for --layer-bench")

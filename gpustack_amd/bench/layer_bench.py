@@ -1,4 +1,4 @@
-"""Layer-level comparison bench: a Vunitar, Fusipel or Livasun stack (`family`) at
+"""Layer-level comparison bench: a Vunitar, Fusipel, Livasun or Makezen stack (`family`) at
 real-model layer sizes beside the closest llama-lineage stack of equal
 width, depth and heads (random weights, synthetic tokens). Reports end-to-end prefill and decode
 throughput through LLMEngine for both, and per-kernel rates of the new
@@ -117,6 +117,50 @@ def livasun_spec(s, moe: bool = False):
         num_heads=1, num_kv_heads=1, head_dim=8, intermediate_size=0,
         rms_norm_eps=1e-5, max_position_embeddings=1 << 20, eos_token_id=-1,
         fp32_residual=True, norm_type="layernorm_bias", embed_scale=4.0)
+
+
+def makezen_spec(s, moe: bool = False):
+    """Layers cycle rotary latent attention (head sizes 128 + 64 rotated,
+    latent 384 — 256 at the small size —, query latent 3/4 of the width,
+    window 1024, sinks, output gates), a gated delta rule (heads x 128 x
+    128, half as many key heads, 4 taps), softmax attention (head size 128,
+    heads/4 kv heads, 64 rotated channels, capped scores) beside a delta
+    rule of half the heads, and latent attention on the first layer's
+    cache; ungated tanh-GELU feed-forward of the llama stack's width."""
+    from ..engine.config import (FeedForwardSpec, LatentMixerSpec, LayerSpec,
+                                 ModelSpec, PagedMixerSpec, ParallelMixerSpec,
+                                 RotarySpec, ScanMixerSpec)
+
+    H, W = s["heads"], s["width"]
+    R = makezen_rank(s)
+    rot = RotarySpec(dims=64, base=10000.0, layout="half",
+                     ramp=(4.0, 4096.0, 32.0, 1.0))
+    lat = dict(heads=H, qk_dim=128, v_dim=128, kv_rank=R,
+               scale=192 ** -0.5, rot_dim=64, rot=rot, q_rank=3 * W // 4,
+               window=1024, sink=True, out_gate=True)
+    delta = ScanMixerSpec(kind="delta", heads=H, state=128, vdim=128,
+                          groups=max(1, H // 2), conv=4)
+    left = PagedMixerSpec(heads=H, kv_heads=max(1, H // 4), qk_dim=128,
+                          v_dim=128, scale=128 ** -0.5, rot=rot, bias=True,
+                          head_norm=True, softcap=30.0)
+    right = ScanMixerSpec(kind="delta", heads=max(1, H // 2), state=128,
+                          vdim=128, groups=max(1, H // 4), conv=4)
+    ff = FeedForwardSpec(kind="dense", ff=s["ff"], act="gelu_tanh")
+    cycle = [("latent_attention", LatentMixerSpec(**lat)), ("scan", delta),
+             ("parallel", ParallelMixerSpec(left=left, right=right)),
+             ("latent_attention", LatentMixerSpec(**lat, kv_from=0))]
+    return ModelSpec(
+        architecture="Makezen", vocab_size=32000, hidden_size=W,
+        num_layers=s["layers"],
+        layers=tuple(LayerSpec(*cycle[i % 4], ff) for i in range(s["layers"])),
+        num_heads=1, num_kv_heads=1, head_dim=8, intermediate_size=0,
+        rms_norm_eps=1e-5, max_position_embeddings=1 << 20, eos_token_id=-1,
+        sandwich_norms=True, fp32_residual=True, norm_type="layernorm",
+        embed_norm=True, tie_word_embeddings=True)
+
+
+def makezen_rank(s) -> int:
+    return 256 if s["width"] <= 1024 else 384
 
 
 def llama_spec(s, moe: bool):
@@ -675,22 +719,255 @@ def livasun_kernel_rates(s, device):
     return out
 
 
+def makezen_kernel_rates(s, device):
+    """Per-kernel rates of the Makezen kernels next to their likes in the
+    Livasun stack (windowed attention, the matrix-state scan and step, its
+    row kernels)."""
+    from .. import ops
+
+    bf = torch.bfloat16
+    H, W, D, BS = s["heads"], s["width"], 128, 16
+    G = max(1, H // 4)
+    R = makezen_rank(s)
+    KW = R + 64
+    out = []
+
+    def rec(name, sec, flops=None, nbytes=None, peak=PEAK_FLOPS):
+        if flops is not None:
+            out.append(dict(kernel=name, us=round(sec * 1e6, 1),
+                            tflops=round(flops / sec / 1e12, 1),
+                            roofline=round(flops / sec / peak, 4)))
+        else:
+            out.append(dict(kernel=name, us=round(sec * 1e6, 1),
+                            gbps=round(nbytes / sec / 1e9, 1),
+                            roofline=round(nbytes / sec / PEAK_BW, 4)))
+
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=device)
+    # ---- prefill attention: 4 prompts x 2048 ----
+    nseq, L, win = 4, 2048, 1024
+    T = nseq * L
+    nblk = T // BS + 1
+    bt = torch.arange(nseq * (L // BS), dtype=torch.int32, device=device).view(nseq, -1)
+    row_seq = torch.arange(nseq, dtype=torch.int32, device=device).repeat_interleave(L)
+    pos = torch.arange(L, dtype=torch.int32, device=device).repeat(nseq)
+    starts = [i * L for i in range(nseq)]
+    wpairs = nseq * sum(min(i + 1, win) for i in range(L))
+    pairs = nseq * L * (L + 1) // 2
+    sinks = torch.zeros(H, device=device)
+    # latent rows: one key "head" of R + 64 channels, values its first R
+    kc = torch.randn(nblk, 1, BS, KW, device=device).to(bf)
+    vc = torch.randn(nblk, 1, R, BS, device=device).to(bf)
+    q_hts = torch.randn(H, T, KW, device=device).to(bf)
+    c_hts = torch.empty(H, T, R, dtype=bf, device=device)
+    tiles = ops.build_attn_tiles(starts, [0] * nseq, [L] * nseq, H, 1, 1, device)
+    rec("paged_attention prefill, latent rows, window 1024 + sink (mfma, useful pairs)",
+        _time(lambda: ops.paged_attention(c_hts.transpose(0, 1),
+                                          q_hts.transpose(0, 1), kc, vc, bt,
+                                          row_seq, pos, 0.07, window=win,
+                                          sinks=sinks, tiles=tiles), 5),
+        flops=2.0 * (KW + R) * H * wpairs)
+    kc = torch.randn(nblk, G, BS, D, device=device).to(bf)
+    vc = torch.randn(nblk, G, D, BS, device=device).to(bf)
+    q = torch.randn(T, H, D, device=device).to(bf)
+    o = torch.empty_like(q)
+    tiles = ops.build_attn_tiles(starts, [0] * nseq, [L] * nseq, H, G, 1, device)
+    rec("paged_attention prefill, causal + score cap (mfma)",
+        _time(lambda: ops.paged_attention(o, q, kc, vc, bt, row_seq, pos,
+                                          D ** -0.5, tiles=tiles, softcap=30.0), 5),
+        flops=4.0 * D * H * pairs)
+    slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / H) for h in range(H)],
+                          device=device)
+    rec("paged_attention prefill, window 1024 + slopes (Livasun, useful pairs)",
+        _time(lambda: ops.paged_attention(o, q, kc, vc, bt, row_seq, pos,
+                                          D ** -0.5, window=win, tiles=tiles,
+                                          slopes=slopes), 5),
+        flops=4.0 * D * H * wpairs)
+
+    # ---- decode attention: 64 sequences x 2048 cached ----
+    B, Lc = 64, 2048
+    nblk = B * (Lc // BS) + 1
+    bt = torch.arange(B * (Lc // BS), dtype=torch.int32, device=device).view(B, -1)
+    row_seq = torch.arange(B, dtype=torch.int32, device=device)
+    pos = torch.full((B,), Lc - 1, dtype=torch.int32, device=device)
+    kc = torch.randn(nblk, 1, BS, KW, device=device).to(bf)
+    vc = torch.randn(nblk, 1, R, BS, device=device).to(bf)
+    q_hts = torch.randn(H, B, KW, device=device).to(bf)
+    c_hts = torch.empty(H, B, R, dtype=bf, device=device)
+    tiles = ops.build_attn_tiles(list(range(B)), [Lc - 1] * B, [1] * B, H, 1, 1,
+                                 device)
+    rec("paged_attention decode, latent rows, window 1024 + sink (mfma)",
+        _time(lambda: ops.paged_attention(c_hts.transpose(0, 1),
+                                          q_hts.transpose(0, 1), kc, vc, bt,
+                                          row_seq, pos, 0.07, window=win,
+                                          sinks=sinks, tiles=tiles, max_ctx=Lc)),
+        nbytes=B * win * (KW + R) * 2)
+    kc = torch.randn(nblk, G, BS, D, device=device).to(bf)
+    vc = torch.randn(nblk, G, D, BS, device=device).to(bf)
+    qd = torch.randn(B, H, D, device=device).to(bf)
+    od = torch.empty_like(qd)
+    tiles = ops.build_attn_tiles(list(range(B)), [Lc - 1] * B, [1] * B, H, G, 1,
+                                 device)
+    rec("paged_attention decode, causal + score cap (mfma)",
+        _time(lambda: ops.paged_attention(od, qd, kc, vc, bt, row_seq, pos,
+                                          D ** -0.5, tiles=tiles, max_ctx=Lc,
+                                          softcap=30.0)),
+        nbytes=B * Lc * G * D * 2 * 2)
+    rec("paged_attention decode, window 1024 + slopes (Livasun)",
+        _time(lambda: ops.paged_attention(od, qd, kc, vc, bt, row_seq, pos,
+                                          D ** -0.5, window=win, tiles=tiles,
+                                          max_ctx=Lc, slopes=slopes)),
+        nbytes=B * win * G * D * 2 * 2)
+
+    # ---- row kernels at T = 8192 ----
+    T = 8192
+    x = torch.randn(T, W, device=device)
+    a = torch.randn(T, W, device=device).to(bf)
+    w32 = torch.ones(W, device=device)
+    hb = torch.empty(T, W, dtype=bf, device=device)
+    rec("sandwich_add_norm, centred (layer norm + add + layer norm, fp32 stream)",
+        _time(lambda: ops.sandwich_add_norm(x, a, w32, 1.0, 1e-5, None, w32, hb,
+                                            center=True)),
+        nbytes=T * W * 12)
+    rec("add_layer_norm (Livasun: add + layer norm)",
+        _time(lambda: ops.add_layer_norm(x, a, w32, w32, 1e-5, hb)),
+        nbytes=T * W * 12)
+    b2 = torch.randn(T, W, device=device).to(bf)
+    rec("dual_rms_mix (two RMS norms, mean)",
+        _time(lambda: ops.dual_rms_mix(hb, a, w32, b2, w32, 1e-5)),
+        nbytes=T * W * 6)
+    nblk = T // BS + 1
+    nq, nk = H * D, G * D
+    kc = torch.zeros(nblk, G, BS, D, dtype=bf, device=device)
+    vc = torch.zeros(nblk, G, D, BS, dtype=bf, device=device)
+    qkv = torch.randn(T, nq + 2 * nk, device=device).to(bf)
+    qo = torch.empty(T, nq, dtype=bf, device=device)
+    wd = torch.ones(D, device=device)
+    inv = torch.tensor([10000.0 ** (-i / 32) for i in range(32)], device=device)
+    slots = torch.arange(T, device=device)
+    p32 = torch.arange(T, dtype=torch.int32, device=device)
+    pg = ops.build_page_groups([0], [0], [T], BS, device)
+    nb_rows = T * (2 * nq + 2 * nk + 2 * nk) * 2      # q, k in/out; v in/out
+    for label, groups in (("values by page", pg), ("values row by row", None)):
+        rec(f"head_rope_store (head norms + rotation + cache write, {label})",
+            _time(lambda: ops.head_rope_store(
+                qo, qkv, 0, H, D, wd, D, 0, nq, G, D, wd, D, 0, nq + nk, inv,
+                True, 1.1, p32, kc, vc, slots, 1e-5, page_groups=groups)),
+            nbytes=nb_rows)
+    vfirst = torch.randn(T, nk, device=device).to(bf)
+    lam = torch.tensor([0.3], device=device)
+    rec("head_norm_store (Livasun: head norms + temperature + blend + cache write, values by page)",
+        _time(lambda: ops.head_norm_store(qo, qkv, nq, nk, wd, wd, D, 0.1, 1024,
+                                          p32, vfirst, lam, kc, vc, slots, 1e-5,
+                                          page_groups=pg)),
+        nbytes=nb_rows + T * nk * 2)
+    # latent rows: query latent normed, latent normed + key part turned,
+    # key row and value pages written
+    QR = 3 * W // 4
+    u = torch.randn(T, QR + KW + H, device=device).to(bf)
+    cq = torch.empty(T, QR, dtype=bf, device=device)
+    kc1 = torch.zeros(nblk, 1, BS, KW, dtype=bf, device=device)
+    vc1 = torch.zeros(nblk, 1, R, BS, dtype=bf, device=device)
+    wq, wr = torch.ones(QR, device=device), torch.ones(R, device=device)
+    rec("head_rope_store, latent rows (two norms + rotation + key row + value pages)",
+        _time(lambda: ops.head_rope_store(
+            cq, u, 0, 1, QR, wq, QR, -1, QR, 1, KW, wr, R, R, -1, inv, True,
+            1.1, p32, kc1, vc1, slots, 1e-5)),
+        nbytes=T * (2 * QR + 2 * KW + R) * 2)
+    qh = torch.randn(T, H * 192, device=device).to(bf)
+    qt = torch.empty_like(qh)
+    rec("head_rope_store, query heads (rotation of the last 64 of 192 channels)",
+        _time(lambda: ops.head_rope_store(
+            qt, qh, 0, H, 192, None, 0, 128, 0, 0, 0, None, 0, -1, -1, inv,
+            True, 1.1, p32, None, None, None, 1e-5)),
+        nbytes=T * H * 192 * 4)
+    o_hts = torch.randn(H, T, D, device=device).to(bf)
+    og = torch.empty(T, H * D, dtype=bf, device=device)
+    rec("head_gate (head-major -> rows, sigmoid gate per head)",
+        _time(lambda: ops.head_gate(og, o_hts, u, QR + KW)),
+        nbytes=T * H * D * 4)
+    uf = torch.randn(T, s["ff"], device=device).to(bf)
+    rec("act_inplace gelu_tanh", _time(lambda: ops.act_inplace(uf, "gelu_tanh")),
+        nbytes=T * s["ff"] * 4)
+    gu = torch.randn(T, 2 * s["ff"], device=device).to(bf)
+    ao = torch.empty(T, s["ff"], dtype=bf, device=device)
+    rec("act_and_mul silu (Livasun)", _time(lambda: ops.act_and_mul(ao, gu, "silu")),
+        nbytes=T * s["ff"] * 6)
+
+    # ---- recurrent mixers: H heads of 128 x 128, H/2 key heads ----
+    N = P = 128
+    Gk, taps = max(1, H // 2), 4
+    nqk, inner = Gk * N, H * P
+    C = 2 * nqk + inner
+    for label, nseq, L in (("prefill 8 x 1024", 8, 1024), ("decode 64 x 1", 64, 1)):
+        T = nseq * L
+        sf, sr = i32([i * L for i in range(nseq)]), i32([L] * nseq)
+        ss = i32(list(range(nseq)))
+        rs = torch.arange(nseq, dtype=torch.int32, device=device).repeat_interleave(L)
+        ps = (torch.arange(L, dtype=torch.int32, device=device) + 5).repeat(nseq)
+        u = torch.randn(T, C + inner + 2 * H, device=device).to(bf)
+        qkv = torch.empty(T, C, dtype=bf, device=device)
+        cw, cb = torch.randn(C, taps, device=device), torch.zeros(C, device=device)
+        cst = torch.zeros(nseq + 1, taps - 1, C, dtype=bf, device=device)
+        rec(f"causal_conv_silu {label}",
+            _time(lambda: ops.causal_conv_silu(qkv, u, 0, cw, cb, cst, sf, sr,
+                                               ss, rs, ps)),
+            nbytes=T * C * 4)
+        y = torch.empty(T, inner, device=device)
+        st = torch.zeros(nseq + 1, H, N, P, device=device)
+        hv = torch.zeros(H, device=device)
+        sec = _time(lambda: ops.delta_scan(y, qkv, 0, nqk, 2 * nqk, u,
+                                           C + inner, C + inner + H, H, Gk, N, P,
+                                           hv - 1, hv, st, sf, sr, ss, ps,
+                                           single=L == 1), 5)
+        if L > 1:
+            rec(f"delta_scan {label} (fp32 vector ALU, 7 flops per state element)",
+                sec, flops=7.0 * T * H * N * P, peak=PEAK_VALU)
+        else:
+            rec(f"delta_scan {label} (state read + write)", sec,
+                nbytes=nseq * H * N * P * 8)
+        ul = torch.randn(T, 4 * H * 128, device=device).to(bf)
+        stl = torch.zeros(nseq + 1, H, 128, 128, device=device)
+        dec = torch.full((H,), 0.99, device=device)
+        sec = _time(lambda: ops.state_scan(y, ul, 2 * H * 128, H * 128, 0, None,
+                                           0, H, H, 128, 128, True, None, None,
+                                           None, dec, stl, sf, sr, ss, ps,
+                                           single=L == 1), 5)
+        if L > 1:
+            rec(f"state_scan lightning {label} (Livasun, 4 flops per state element)",
+                sec, flops=4.0 * T * H * 128 * 128, peak=PEAK_VALU)
+        else:
+            rec(f"state_scan lightning {label} (Livasun, state read + write)",
+                sec, nbytes=nseq * H * 128 * 128 * 8)
+        g = torch.empty(T, inner, dtype=bf, device=device)
+        wi = torch.ones(inner, device=device)
+        rec(f"gated_group_norm per head, SiLU gate {label}",
+            _time(lambda: ops.gated_group_norm(g, y, u[:, C:C + inner], wi, H,
+                                               1e-5, 2)),
+            nbytes=T * inner * 8)
+    return out
+
+
 def run(sizes: list[str], device: str, family: str = "vunitar") -> None:
     for name in sizes:
         s = SIZES[name]
-        if family == "livasun":
-            s = dict(s, layers=4)       # one full cycle of the three mixers
+        if family in ("livasun", "makezen"):
+            s = dict(s, layers=4)       # one full cycle of the mixers
         for moe in ((False, True) if family in ("vunitar", "livasun")
                     else (False,)):
             row = {"size": name, **s, "ff_kind": "moe" if moe else "dense"}
             mine = {"vunitar": vunitar_spec, "fusipel": fusipel_spec,
-                    "livasun": livasun_spec}[family]
-            for label, mk in ((family, mine), ("llama_graph", llama_spec)):
+                    "livasun": livasun_spec, "makezen": makezen_spec}[family]
+            # Makezen's closest existing model is the other hybrid of
+            # attention and recurrent layers; the llama graph for scale
+            others = ((("livasun", livasun_spec),) if family == "makezen"
+                      else ()) + (("llama_graph", llama_spec),)
+            for label, mk in ((family, mine),) + others:
                 pre, dec = engine_rates(mk(s, moe), device)
                 row[label] = {"prefill_tok_s": round(pre), "decode_tok_s": round(dec)}
             print(json.dumps({"layer_bench": row}), flush=True)
         if torch.cuda.is_available():
             rates = {"vunitar": kernel_rates, "fusipel": fusipel_kernel_rates,
-                     "livasun": livasun_kernel_rates}[family]
+                     "livasun": livasun_kernel_rates,
+                     "makezen": makezen_kernel_rates}[family]
             for k in rates(s, device):
                 print(json.dumps({"kernel_bench": {"size": name, **k}}), flush=True)

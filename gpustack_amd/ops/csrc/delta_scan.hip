@@ -178,6 +178,198 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(
   }
 }
 
+
+// The same recurrence for bf16 sources whose sizes and columns are multiples
+// of 8: four waves share one (sequence, head) and 4 * PL value channels, so
+// k and q are staged once for all of them with 16-byte loads; the next CH
+// rows are fetched into registers while the current ones are walked (two LDS
+// buffers). A lane owns the state rows ns * NR .. ns * NR + NR - 1 and reads
+// its k / q slice from LDS in 16-byte pieces; slices of different ns sit
+// NR + 4 floats apart, on other banks. The lengths of k and q and their
+// product are summed from the staged rows, 16 lanes per row.
+constexpr int CH = 16;     // rows staged per pass
+
+template <int NR, int TPP>
+__global__ __launch_bounds__(256) void delta_scan_vec_kernel(
+    float* __restrict__ y, const unsigned short* __restrict__ src,
+    const unsigned short* __restrict__ gate_src, DeltaArgs p) {
+  constexpr int PL = 64 / TPP;
+  constexpr int NP = NR * TPP;
+  constexpr int NS = NR + 4;                 // floats between two ns slices
+  constexpr int ROW = TPP * NS;              // floats per staged k / q row
+  constexpr int PB = 4 * PL;                 // value channels per workgroup
+  constexpr int KV = (CH * NP / 8 + 255) / 256;   // 16-byte loads per lane
+  constexpr int VV = (CH * PB / 8 + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float ks[2][CH][ROW];
+  __shared__ __attribute__((aligned(16))) float qs[2][CH][ROW];
+  __shared__ float vs[2][CH][PB];
+  __shared__ float g_s[2][CH], b_s[2][CH], ck_s[2][CH], cq_s[2][CH], kq_s[2][CH];
+  const int s = blockIdx.x, h = blockIdx.y, pb0 = blockIdx.z * PB;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int pl = lane % PL, ns = lane / PL;
+  const int first = p.seq_first[s], n = p.seq_rows[s];
+  if (first < 0 || n < 1 || first + n > p.T) return;
+  const int slot = min(max(p.state_slots[s], 0), p.nslots - 1);
+  const int hist = p.pos32[first];
+  const int N = p.N, P = p.P;
+  const int g = h / (p.H / p.G);
+  const int pc = pb0 + wave * PL + pl;
+  const bool live = pc < P;
+  float* sp = p.state + ((long)slot * p.H + h) * N * P;
+  float S[NR];
+#pragma unroll
+  for (int j = 0; j < NR; ++j) {
+    const int nn = ns * NR + j;
+    S[j] = (hist > 0 && live && nn < N) ? sp[(long)nn * P + pc] : 0.f;
+  }
+  const float a_rate = expf(p.a_log[h]);
+  const float dtb = p.dt_bias[h];
+  const int nvec = N / 8;                    // 16-byte pieces per k / q row
+  const u16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  u16x8 kreg[KV], qreg[KV], vreg[VV];
+  float areg = 0.f, breg = 0.f;
+  auto fetch = [&](int c0) {
+    const int rows = min(CH, n - c0);
+#pragma unroll
+    for (int u = 0; u < KV; ++u) {
+      const int i = tid + u * 256;
+      kreg[u] = zero8;
+      qreg[u] = zero8;
+      if (i < rows * nvec) {
+        const int r = i / nvec, e = (i % nvec) * 8;
+        const unsigned short* rp = src + (long)(first + c0 + r) * p.ld_src;
+        kreg[u] = *reinterpret_cast<const u16x8*>(rp + p.col_k + g * N + e);
+        qreg[u] = *reinterpret_cast<const u16x8*>(rp + p.col_q + g * N + e);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < VV; ++u) {
+      const int i = tid + u * 256;
+      vreg[u] = zero8;
+      if (i < rows * (PB / 8)) {
+        const int r = i / (PB / 8), c = (i % (PB / 8)) * 8;
+        if (pb0 + c < P)
+          vreg[u] = *reinterpret_cast<const u16x8*>(
+              src + (long)(first + c0 + r) * p.ld_src + p.col_v + h * P + pb0 + c);
+      }
+    }
+    if (tid < rows) {
+      const unsigned short* gp = gate_src + (long)(first + c0 + tid) * p.ld_gate;
+      areg = bf2f(gp[p.col_a + h]);
+      breg = bf2f(gp[p.col_b + h]);
+    }
+  };
+  auto stage = [&](int buf, int c0) {
+    const int rows = min(CH, n - c0);
+#pragma unroll
+    for (int u = 0; u < KV; ++u) {
+      const int i = tid + u * 256;
+      if (i < rows * nvec) {
+        const int r = i / nvec, e = (i % nvec) * 8;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const int nn = e + k;
+          const int at = (nn / NR) * NS + nn % NR;
+          ks[buf][r][at] = bf2f(kreg[u][k]);
+          qs[buf][r][at] = bf2f(qreg[u][k]);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < VV; ++u) {
+      const int i = tid + u * 256;
+      if (i < rows * (PB / 8)) {
+        const int r = i / (PB / 8), c = (i % (PB / 8)) * 8;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) vs[buf][r][c + k] = bf2f(vreg[u][k]);
+      }
+    }
+    if (tid < rows) {
+      const float dt = softplus_f(areg + dtb);
+      g_s[buf][tid] = expf(-a_rate * dt);
+      b_s[buf][tid] = 1.0f / (1.0f + expf(-breg));
+    }
+  };
+  // state rows past N (padding up to NP) keep k = q = 0: zero them once
+  for (int i = tid; i < 2 * CH * ROW; i += 256) {
+    (&ks[0][0][0])[i] = 0.f;
+    (&qs[0][0][0])[i] = 0.f;
+  }
+  __syncthreads();
+  fetch(0);
+  int buf = 0;
+  for (int c0 = 0; c0 < n; c0 += CH, buf ^= 1) {
+    const int rows = min(CH, n - c0);
+    stage(buf, c0);
+    __syncthreads();
+    {
+      // 16 lanes per staged row: sum over the padded row (zeros add nothing)
+      const int r = tid >> 4, sub = tid & 15;
+      float kk = 0.f, qq = 0.f, kq = 0.f;
+      for (int i = sub; i < ROW; i += 16) {
+        const float kv = ks[buf][r][i], qv = qs[buf][r][i];
+        kk += kv * kv;
+        qq += qv * qv;
+        kq += kv * qv;
+      }
+#pragma unroll
+      for (int m = 8; m >= 1; m >>= 1) {
+        kk += __shfl_xor(kk, m, WAVE_SIZE);
+        qq += __shfl_xor(qq, m, WAVE_SIZE);
+        kq += __shfl_xor(kq, m, WAVE_SIZE);
+      }
+      if (sub == 0) {
+        const float ck = 1.0f / sqrtf(kk + 1e-6f);
+        const float cq = p.q_scale / sqrtf(qq + 1e-6f);
+        ck_s[buf][r] = ck;
+        cq_s[buf][r] = cq;
+        kq_s[buf][r] = ck * cq * kq;
+      }
+    }
+    __syncthreads();
+    if (c0 + CH < n) fetch(c0 + CH);
+    const float* kb = &ks[buf][0][ns * NS];
+    const float* qb = &qs[buf][0][ns * NS];
+    for (int r = 0; r < rows; ++r) {
+      const float a = g_s[buf][r];
+      float dk = 0.f, dq = 0.f;
+      f32x4 k4[NR / 4];
+#pragma unroll
+      for (int j = 0; j < NR; j += 4) {
+        k4[j / 4] = *reinterpret_cast<const f32x4*>(kb + r * ROW + j);
+        const f32x4 q4 = *reinterpret_cast<const f32x4*>(qb + r * ROW + j);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          S[j + k] *= a;
+          dk += S[j + k] * k4[j / 4][k];
+          dq += S[j + k] * q4[k];
+        }
+      }
+#pragma unroll
+      for (int m = PL; m < 64; m <<= 1) {
+        dk += __shfl_xor(dk, m, WAVE_SIZE);
+        dq += __shfl_xor(dq, m, WAVE_SIZE);
+      }
+      const float ck = ck_s[buf][r];
+      const float u = b_s[buf][r] * (vs[buf][r][wave * PL + pl] - ck * dk);
+      const float cu = ck * u;
+#pragma unroll
+      for (int j = 0; j < NR; j += 4)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) S[j + k] += k4[j / 4][k] * cu;
+      if (ns == 0 && live)
+        y[(long)(first + c0 + r) * p.H * P + h * P + pc] =
+            cq_s[buf][r] * dq + u * kq_s[buf][r];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < NR; ++j) {
+    const int nn = ns * NR + j;
+    if (live && nn < N) sp[(long)nn * P + pc] = S[j];
+  }
+}
+
 DEVICE_INLINE float block_sum3(float v, float* red, int slot) {
   v = wave_reduce_sum(v);
   if ((threadIdx.x & 63) == 0) red[slot * 4 + (threadIdx.x >> 6)] = v;
@@ -323,11 +515,25 @@ bool delta_pick(float* y, const void* src, const void* gate,
   while (tpp < 8 && (p.N + tpp - 1) / tpp >= 16 &&
          (long)nseq * p.H * ((p.P + 64 / tpp - 1) / (64 / tpp)) < 1024)
     tpp *= 2;
+  // 16-byte staging: bf16 rows whose sizes and columns are multiples of 8
+  const bool vec = sizeof(TS) == 2 && p.N % 8 == 0 && p.P % 8 == 0 &&
+                   p.ld_src % 8 == 0 && p.col_q % 8 == 0 && p.col_k % 8 == 0 &&
+                   p.col_v % 8 == 0;
   const int nr = (p.N + tpp - 1) / tpp;
-#define DELTA_CASE(NRV, TPPV)                                   \
-  if (tpp == TPPV && nr <= NRV) {                               \
-    delta_launch<TS, NRV, TPPV>(y, src, gate, p, nseq, s);      \
-    return true;                                                \
+#define DELTA_CASE(NRV, TPPV)                                                \
+  if (tpp == TPPV && nr <= NRV) {                                            \
+    constexpr bool fits = sizeof(TS) == 2 && NRV % 4 == 0 &&                 \
+        (4 * CH * TPPV * (NRV + 4) + 2 * CH * 4 * (64 / TPPV) + 10 * CH) * 4 \
+            <= 60 * 1024;                                                    \
+    if constexpr (fits) if (vec) {                                           \
+      constexpr int PBV = 4 * (64 / TPPV);                                   \
+      dim3 grid(nseq, p.H, (p.P + PBV - 1) / PBV);                           \
+      delta_scan_vec_kernel<NRV, TPPV><<<grid, 256, 0, s>>>(                 \
+          y, (const unsigned short*)src, (const unsigned short*)gate, p);    \
+      return true;                                                           \
+    }                                                                        \
+    delta_launch<TS, NRV, TPPV>(y, src, gate, p, nseq, s);                   \
+    return true;                                                             \
   }
 #define DELTA_TPP(TPPV) \
   DELTA_CASE(4, TPPV) DELTA_CASE(8, TPPV) DELTA_CASE(16, TPPV) DELTA_CASE(32, TPPV)

@@ -204,8 +204,10 @@ void paged_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
   TORCH_CHECK((maps == 1 || maps == 2) && A % maps == 0 && KW == maps * D);
   const int H = A / maps;
   TORCH_CHECK(G >= 1 && H % G == 0, "heads must be a multiple of kv heads");
-  TORCH_CHECK(D >= 1 && D <= paged_attn_max_dim() && VW >= 1 &&
-              VW <= paged_attn_max_dim(), "head size unsupported");
+  const bool mfma = !exact && paged_attn_uses_mfma(q_bf, BS, D, VW);
+  TORCH_CHECK(D >= 1 && VW >= 1 &&
+              (mfma || (D <= paged_attn_max_dim() && VW <= paged_attn_max_dim())),
+              "head size unsupported");
   TORCH_CHECK(block_tables.dim() == 2 && block_tables.size(1) >= 1 &&
               tiles.dim() == 2 && tiles.size(1) == 6 && pos32.numel() == T);
   TORCH_CHECK(window >= 0 && keep_first >= 0);
@@ -221,7 +223,6 @@ void paged_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
     TORCH_CHECK(slopes->numel() == H);
     slp = slopes->data_ptr<float>();
   }
-  const bool mfma = !exact && paged_attn_uses_mfma(q_bf, BS, D, VW);
   if (!mfma) nsplit = 1;
   TORCH_CHECK(nsplit >= 1 && nsplit <= 64);
   const int ntiles = tiles.size(0);

@@ -520,7 +520,8 @@ void dispatch_mfma(void* out, const void* q, const void* kc, const void* vc,
   const int nt = (p.VW / 16 + 3) / 4;
   if (nt <= 1) launch_mfma<1, TO>(out, q, kc, vc, p, ntiles, nsplit, ws_acc, ws_ml, s);
   else if (nt <= 2) launch_mfma<2, TO>(out, q, kc, vc, p, ntiles, nsplit, ws_acc, ws_ml, s);
-  else launch_mfma<4, TO>(out, q, kc, vc, p, ntiles, nsplit, ws_acc, ws_ml, s);
+  else if (nt <= 4) launch_mfma<4, TO>(out, q, kc, vc, p, ntiles, nsplit, ws_acc, ws_ml, s);
+  else launch_mfma<8, TO>(out, q, kc, vc, p, ntiles, nsplit, ws_acc, ws_ml, s);
 }
 
 template <typename TQ, typename TC, typename TO, int NJ, int KT>
@@ -558,13 +559,14 @@ void dispatch_exact(void* out, const void* q, const void* kc, const void* vc,
 
 }  // namespace
 
-// largest head sizes the exact path's LDS tiling covers
+// largest head sizes the exact path's LDS tiling covers (the MFMA path
+// takes score sizes up to 1024 and value sizes up to 512)
 int paged_attn_max_dim() { return 512; }
 
 // 1 when (q / pool dtype, page size, head sizes) take the MFMA path
 int paged_attn_uses_mfma(int io_bf, int BS, int D, int VW) {
-  return io_bf && BS == 16 && D % 32 == 0 && D <= 512 && VW % 16 == 0 &&
-         VW <= 256;
+  return io_bf && BS == 16 && D % 32 == 0 && D <= 1024 && VW % 16 == 0 &&
+         VW <= 512;
 }
 
 // q_bf: q and the pools are bf16, else fp32. out_bf: out is bf16, else fp32.

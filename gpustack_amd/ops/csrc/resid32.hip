@@ -298,6 +298,33 @@ __global__ void act_inplace_kernel(T* __restrict__ x, long n, int mode) {
     st(x + i, act_apply(ld(x + i), mode));
 }
 
+// bf16, n % 8 == 0: 16 bytes per lane. The tanh form of GELU is
+// z * sigmoid(2u), one exponential per element.
+template <int MODE>
+__global__ __launch_bounds__(256) void act_inplace_vec_kernel(
+    unsigned short* __restrict__ x, long n8) {
+  const long stride = (long)gridDim.x * blockDim.x;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += stride) {
+    const u16x8 v = reinterpret_cast<const u16x8*>(x)[i];
+    u16x8 o;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float z = bf2f(v[k]);
+      float r;
+      if (MODE == 2) {
+        const float u = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+        r = z / (1.0f + __expf(-2.0f * u));
+      } else if (MODE == 3) {
+        r = z / (1.0f + __expf(-z));
+      } else {
+        r = act_apply(z, MODE);
+      }
+      o[k] = f2bf(r);
+    }
+    reinterpret_cast<u16x8*>(x)[i] = o;
+  }
+}
+
 __global__ void softcap_kernel(float* __restrict__ x, long n, float cap) {
   const long stride = (long)gridDim.x * blockDim.x;
   const float inv = 1.0f / cap;
@@ -514,6 +541,18 @@ void latent_norm_store_launch(void* cache, const void* src, long ld_src,
 void act_inplace_launch(void* x, long n, int mode, int bf, hipStream_t s) {
   if (n == 0) return;
   const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+  if (bf && n % 8 == 0 && ((uintptr_t)x % 16) == 0) {
+    const long n8 = n / 8;
+    const int b8 = (int)((n8 + 255) / 256 < 16384 ? (n8 + 255) / 256 : 16384);
+    auto* xp = (unsigned short*)x;
+    switch (mode) {
+      case 0: act_inplace_vec_kernel<0><<<b8, 256, 0, s>>>(xp, n8); break;
+      case 1: act_inplace_vec_kernel<1><<<b8, 256, 0, s>>>(xp, n8); break;
+      case 2: act_inplace_vec_kernel<2><<<b8, 256, 0, s>>>(xp, n8); break;
+      default: act_inplace_vec_kernel<3><<<b8, 256, 0, s>>>(xp, n8); break;
+    }
+    return;
+  }
   if (bf)
     act_inplace_kernel<unsigned short><<<blocks, 256, 0, s>>>(
         (unsigned short*)x, n, mode);

@@ -182,6 +182,90 @@ __global__ __launch_bounds__(ROW_THREADS) void dual_rms_mix_kernel(
        0.5f * (ld(ar + i) * ia * wa[i] + ld(br + i) * ib * wb[i]));
 }
 
+// W % 4 == 0 and W <= NV * 1024: four consecutive channels per lane and step,
+// both rows in registers between the sums of squares and the store.
+template <typename T> struct V4;
+template <> struct V4<float> {
+  static DEVICE_INLINE void load(const float* p, float* o) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(p);
+    o[0] = v[0]; o[1] = v[1]; o[2] = v[2]; o[3] = v[3];
+  }
+  static DEVICE_INLINE void store(float* p, const float* o) {
+    *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
+  }
+};
+template <> struct V4<unsigned short> {
+  static DEVICE_INLINE void load(const unsigned short* p, float* o) {
+    const u16x4 v = *reinterpret_cast<const u16x4*>(p);
+    o[0] = bf2f(v[0]); o[1] = bf2f(v[1]); o[2] = bf2f(v[2]); o[3] = bf2f(v[3]);
+  }
+  static DEVICE_INLINE void store(unsigned short* p, const float* o) {
+    *reinterpret_cast<u16x4*>(p) = u16x4{f2bf(o[0]), f2bf(o[1]), f2bf(o[2]), f2bf(o[3])};
+  }
+};
+
+template <typename TS, int NV>
+__global__ __launch_bounds__(ROW_THREADS) void dual_rms_mix_vec_kernel(
+    TS* __restrict__ out, const TS* __restrict__ a, const float* __restrict__ wa,
+    const TS* __restrict__ b, const float* __restrict__ wb, int W, float eps) {
+  __shared__ float red[4];
+  const long t = blockIdx.x;
+  float ka[NV][4], kb[NV][4];
+  float sa = 0.f, sb = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int i = (threadIdx.x + j * ROW_THREADS) * 4;
+    if (i < W) {
+      V4<TS>::load(a + t * W + i, ka[j]);
+      V4<TS>::load(b + t * W + i, kb[j]);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        sa += ka[j][k] * ka[j][k];
+        sb += kb[j][k] * kb[j][k];
+      }
+    }
+  }
+  sa = block_sum(sa, red);
+  sb = block_sum(sb, red);
+  const float ia = 0.5f / sqrtf(sa / (float)W + eps);
+  const float ib = 0.5f / sqrtf(sb / (float)W + eps);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int i = (threadIdx.x + j * ROW_THREADS) * 4;
+    if (i < W) {
+      float x[4], yv[4], o[4];
+      V4<float>::load(wa + i, x);
+      V4<float>::load(wb + i, yv);
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        o[k] = ka[j][k] * ia * x[k] + kb[j][k] * ib * yv[k];
+      V4<TS>::store(out + t * W + i, o);
+    }
+  }
+}
+
+// bf16, VD % 8 == 0: 16 bytes per lane.
+__global__ __launch_bounds__(256) void head_gate_vec_kernel(
+    unsigned short* __restrict__ out, const unsigned short* __restrict__ o_hts,
+    const unsigned short* __restrict__ gate_src, long ld_gate, int col, int H,
+    int T, int VD8) {
+  const long n = (long)T * H * VD8;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long)gridDim.x * blockDim.x) {
+    const int c = (int)(i % VD8);
+    const long th = i / VD8;
+    const int h = (int)(th % H);
+    const long t = th / H;
+    const float g = bf2f(gate_src[t * ld_gate + col + h]);
+    const float sg = 1.0f / (1.0f + __expf(-g));
+    const u16x8 v = reinterpret_cast<const u16x8*>(o_hts)[((long)h * T + t) * VD8 + c];
+    u16x8 o;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) o[k] = f2bf(bf2f(v[k]) * sg);
+    reinterpret_cast<u16x8*>(out)[i] = o;
+  }
+}
+
 template <typename TS>
 __global__ __launch_bounds__(256) void head_gate_kernel(
     TS* __restrict__ out, const TS* __restrict__ o_hts,
@@ -236,6 +320,24 @@ void dual_rms_mix_launch(void* out, const void* a, const float* wa,
                          const void* b, const float* wb, int T, int W,
                          float eps, int bf, hipStream_t s) {
   if (T <= 0) return;
+  if (W % 4 == 0 && W <= 8 * 1024) {
+#define DRV(TS, NV)                                                         \
+  dual_rms_mix_vec_kernel<TS, NV><<<T, ROW_THREADS, 0, s>>>(                \
+      (TS*)out, (const TS*)a, wa, (const TS*)b, wb, W, eps)
+    if (bf) {
+      if (W <= 1024) DRV(unsigned short, 1);
+      else if (W <= 2048) DRV(unsigned short, 2);
+      else if (W <= 4096) DRV(unsigned short, 4);
+      else DRV(unsigned short, 8);
+    } else {
+      if (W <= 1024) DRV(float, 1);
+      else if (W <= 2048) DRV(float, 2);
+      else if (W <= 4096) DRV(float, 4);
+      else DRV(float, 8);
+    }
+#undef DRV
+    return;
+  }
 #define DRM(TS, NV)                                                         \
   dual_rms_mix_kernel<TS, NV><<<T, ROW_THREADS, 0, s>>>(                    \
       (TS*)out, (const TS*)a, wa, (const TS*)b, wb, W, eps)
@@ -255,6 +357,13 @@ void head_gate_launch(void* out, const void* o_hts, const void* gate_src,
   const long n = (long)T * H * VD;
   if (n <= 0) return;
   const int grid = (int)min((n + 255) / 256, (long)(256 * 32));
+  if (bf && VD % 8 == 0) {
+    const int g8 = (int)min((n / 8 + 255) / 256, (long)(256 * 32));
+    head_gate_vec_kernel<<<g8, 256, 0, s>>>(
+        (unsigned short*)out, (const unsigned short*)o_hts,
+        (const unsigned short*)gate_src, ld_gate, col, H, T, VD / 8);
+    return;
+  }
   if (bf)
     head_gate_kernel<unsigned short><<<grid, 256, 0, s>>>(
         (unsigned short*)out, (const unsigned short*)o_hts,

@@ -144,7 +144,11 @@ def test_delta_scan(dtype, H, G, N, P, single):
     else:
         news, hists = [19, 1, 40], [0, 5, 33]
     T, nseq = sum(news), len(news)
-    src = torch.randn(T, 2 * nqk + H * P + 3, generator=g).to(dtype)
+    # sizes of a multiple of 8 sit at columns of a multiple of 8 in rows of
+    # a multiple of 8, which is what the 16-byte staging kernel asks for
+    off = 8 if N % 8 == 0 and P % 8 == 0 else 1
+    width = off + 2 * nqk + H * P + 3
+    src = torch.randn(T, width + (-width) % 8, generator=g).to(dtype)
     gates = (torch.randn(T, 2 * H + 2, generator=g) * 2).to(dtype)
     dt_bias = torch.randn(H, generator=g)
     a_log = torch.randn(H, generator=g) - 1
@@ -160,8 +164,8 @@ def test_delta_scan(dtype, H, G, N, P, single):
         st = state0.clone().to(dev)
         fn = ops.delta_scan if dev == "cuda" else torch_ref.delta_scan
         kw_ = {"single": single} if dev == "cuda" else {}
-        fn(y, to(src), 1, 1 + nqk, 1 + 2 * nqk, to(gates), 1, 1 + H, H, G, N,
-           P, to(dt_bias), to(a_log), st, to(meta(first)), to(meta(news)),
+        fn(y, to(src), off, off + nqk, off + 2 * nqk, to(gates), 1, 1 + H, H,
+           G, N, P, to(dt_bias), to(a_log), st, to(meta(first)), to(meta(news)),
            to(slots), to(pos), **kw_)
         return y, st
 
@@ -220,17 +224,19 @@ def test_head_gate(dtype):
 
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("exact", [False, True])
-def test_paged_attention_cap_window_sink_on_strided_views(dtype, exact):
+@pytest.mark.parametrize("D,VW", [(64, 32), (448, 384)])
+def test_paged_attention_cap_window_sink_on_strided_views(dtype, exact, D, VW):
     """Multi-query attention on head-major q / out buffers handed over as
-    [T, heads, *] views, with a window, sinks and a score cap."""
+    [T, heads, *] views, with a window, sinks and a score cap; also at a
+    latent row's sizes (value channels beyond 256)."""
     g = torch.Generator().manual_seed(5)
-    H, D, VW, BS = 6, 64, 32, 16
+    H, BS = 6, 16
     starts, hists, news = [0, 30], [50, 0], [30, 9]
     T = 39
     nb = 8
     kc = torch.randn(nb, 1, BS, D, generator=g).to(dtype)
     vc = torch.randn(nb, 1, VW, BS, generator=g).to(dtype)
-    q_hts = torch.randn(H, T, D, generator=g).to(dtype)
+    q_hts = (torch.randn(H, T, D, generator=g) * (64.0 / D) ** 0.5).to(dtype)
     bt = torch.tensor([[2, 5, 1, 7, 3], [4, 0, 6, 0, 0]], dtype=torch.int32)
     row_seq = torch.tensor([0] * 30 + [1] * 9, dtype=torch.int32)
     pos = torch.tensor(list(range(50, 80)) + list(range(9)), dtype=torch.int32)
