@@ -64,6 +64,9 @@ def parse_args():
     ap.add_argument("--layer-family", default="vunitar",
                     choices=["vunitar", "fusipel", "livasun", "makezen"],
                     help="model family measured by --layer-bench")
+    ap.add_argument("--layer-solo", action="store_true",
+                    help="--layer-bench: only the family's own stack end to "
+                         "end (the run to put under a profiler)")
     ap.add_argument("--layer-sizes", default="small,medium",
                     help="comma list of small,medium,large for --layer-bench")
     return ap.parse_args()
@@ -77,7 +80,7 @@ def main():
         run_layer_bench(args.layer_sizes.split(","),
                         args.device or ("cuda:0" if torch.cuda.is_available()
                                         else "cpu"),
-                        family=args.layer_family)
+                        family=args.layer_family, solo=args.layer_solo)
         return
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))

@@ -947,7 +947,10 @@ def makezen_kernel_rates(s, device):
     return out
 
 
-def run(sizes: list[str], device: str, family: str = "vunitar") -> None:
+def run(sizes: list[str], device: str, family: str = "vunitar",
+        solo: bool = False) -> None:
+    """`solo`: only the family's own stack end to end (no comparison stack,
+    no per-kernel rates) — the run to put under a profiler."""
     for name in sizes:
         s = SIZES[name]
         if family in ("livasun", "makezen"):
@@ -961,11 +964,11 @@ def run(sizes: list[str], device: str, family: str = "vunitar") -> None:
             # attention and recurrent layers; the llama graph for scale
             others = ((("livasun", livasun_spec),) if family == "makezen"
                       else ()) + (("llama_graph", llama_spec),)
-            for label, mk in ((family, mine),) + others:
+            for label, mk in ((family, mine),) + (() if solo else others):
                 pre, dec = engine_rates(mk(s, moe), device)
                 row[label] = {"prefill_tok_s": round(pre), "decode_tok_s": round(dec)}
             print(json.dumps({"layer_bench": row}), flush=True)
-        if torch.cuda.is_available():
+        if torch.cuda.is_available() and not solo:
             rates = {"vunitar": kernel_rates, "fusipel": fusipel_kernel_rates,
                      "livasun": livasun_kernel_rates,
                      "makezen": makezen_kernel_rates}[family]

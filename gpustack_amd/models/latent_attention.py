@@ -155,6 +155,9 @@ class RotaryLatentAttention(nn.Module):
         amp = m.rot.amplitude
         u = F.linear(h, self.in_w)
         cq = torch.empty(T, self.qr, dtype=h.dtype, device=h.device)
+        groups = (rg.page_groups(k_cache.shape[2])
+                  if self.own_kv and h.is_cuda and k_cache.shape[2] == 16
+                  else None)
         # query latent normed; latent normed + key part turned -> the pool.
         # This step's rows are read back from the pool like older ones
         ops.head_rope_store(
@@ -163,7 +166,8 @@ class RotaryLatentAttention(nn.Module):
             self.r, self.r, -1, self.inv_freq, half, amp, rg.pos32,
             k_cache if self.own_kv else None,
             v_cache if self.own_kv else None,
-            meta.slot_mapping if self.own_kv else None, self.eps)
+            meta.slot_mapping if self.own_kv else None, self.eps,
+            page_groups=groups)
         qh = F.linear(cq, self.uq_w)                          # [T, H*(dq+rd)]
         qt = torch.empty_like(qh)
         ops.head_rope_store(

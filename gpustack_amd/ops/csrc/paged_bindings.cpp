@@ -9,7 +9,7 @@
 void embed_rows_f32_launch(float*, const long*, const void*, int, int, long, int, hipStream_t);
 void sandwich_add_norm_launch(float*, const void*, const float*, float, const float*, const float*, void*, int, int, float, int, int, int, hipStream_t);
 void rotary_norm_store_launch(void*, const void*, long, int, int, int, const float*, const float*, const float*, int, const int*, int, void*, void*, const long*, long, int, int, int, int, float, int, int, int, hipStream_t);
-void value_page_store_launch(const void*, long, int, void*, const long*, long, const int*, int, int, int, int, int, hipStream_t);
+void value_page_store_launch(const void*, long, int, void*, const long*, long, const int*, int, int, int, int, int, int, hipStream_t);
 void diff_combine_launch(void*, const float*, const float*, float, float, long, int, int, hipStream_t);
 void act_and_mul_launch(void*, const void*, long, int, int, int, hipStream_t);
 void argmax_f32_launch(long*, const float*, int, int, hipStream_t);
@@ -173,7 +173,7 @@ void rotary_norm_store(Tensor q_out, Tensor qkv, long nq, long nk,
                             (int)(tied ? nq : nq + nk), v_cache.data_ptr(),
                             slots.data_ptr<long>(), k_cache.size(0) * (long)BS,
                             page_groups->data_ptr<int>(),
-                            (int)page_groups->size(0), T, G, VW, bf,
+                            (int)page_groups->size(0), T, G, VW, bf, 0,
                             cur_stream(qkv));
     HIP_CHECK_LAST();
   }
@@ -347,7 +347,11 @@ void head_rope_store(OptTensor q_out, Tensor src, long col_q, long q_heads,
     sp = slots->data_ptr<long>();
     nslots = k_cache->size(0) * (long)BS;
   }
-  const bool by_page = page_groups.has_value() && k_heads > 0 && col_v >= 0;
+  // values page by page: from the projection's value columns, or — one key
+  // head whose first channels are the values — from the key pool's rows
+  // this launch has just written
+  const bool by_page = page_groups.has_value() && k_heads > 0 &&
+                       (col_v >= 0 || k_heads == 1);
   head_rope_store_launch(
       qp, src.data_ptr(), src.stride(0), (int)col_q, (int)q_heads, (int)q_dim,
       q_w.has_value() && q_heads > 0 ? q_w->data_ptr<float>() : nullptr,
@@ -362,10 +366,16 @@ void head_rope_store(OptTensor q_out, Tensor src, long col_q, long q_heads,
     chk(*page_groups, "page_groups", at::kInt);
     TORCH_CHECK(BS == 16, "page-wise value stores need 16-token pages");
     TORCH_CHECK(page_groups->dim() == 2 && page_groups->size(1) == 2);
-    value_page_store_launch(src.data_ptr(), src.stride(0), (int)col_v, vp, sp,
-                            nslots, page_groups->data_ptr<int>(),
-                            (int)page_groups->size(0), T, (int)k_heads, VW, bf,
-                            cur_stream(src));
+    if (col_v >= 0)
+      value_page_store_launch(src.data_ptr(), src.stride(0), (int)col_v, vp,
+                              sp, nslots, page_groups->data_ptr<int>(),
+                              (int)page_groups->size(0), T, (int)k_heads, VW,
+                              bf, 0, cur_stream(src));
+    else
+      value_page_store_launch(kp, k_dim, 0, vp, sp, nslots,
+                              page_groups->data_ptr<int>(),
+                              (int)page_groups->size(0), T, 1, VW, bf, 1,
+                              cur_stream(src));
     HIP_CHECK_LAST();
   }
 }

@@ -122,7 +122,7 @@ __global__ __launch_bounds__(ROW_THREADS) void head_rope_store_kernel(
       st(q_out + ((long)t * p.q_heads + hd) * dim + c, v);
     } else {
       st(k_cache + ((blk * G + hd) * p.BS + off) * (long)dim + c, v);
-      if (p.col_v < 0 && c < p.VW)
+      if (p.col_v < 0 && !p.skip_v && c < p.VW)
         st(v_cache + ((blk * G + hd) * (long)p.VW + c) * p.BS + off, v);
     }
   }
@@ -130,6 +130,134 @@ __global__ __launch_bounds__(ROW_THREADS) void head_rope_store_kernel(
     const TS* vs = src + (long)t * p.ld_src + p.col_v + (long)hd * p.VW;
     for (int c = lane; c < p.VW; c += 64)
       v_cache[((blk * G + hd) * (long)p.VW + c) * p.BS + off] = vs[c];
+  }
+}
+
+
+// bf16 with every size, column and rotation boundary a multiple of 8: a lane
+// takes 8 consecutive channels of its head (16 bytes) per step, LPH lanes
+// share a head (the smallest power of two that covers the widest head in
+// one step, at most a wave) and a wave takes 64 / LPH heads. A rotated piece
+// in the (i, i + half) layout fetches its partner piece as well, in the
+// (2i, 2i + 1) layout the partners sit in the same piece.
+template <int LPH>
+__global__ __launch_bounds__(ROW_THREADS) void head_rope_store_vec_kernel(
+    unsigned short* __restrict__ q_out, const unsigned short* __restrict__ src,
+    unsigned short* __restrict__ k_cache, unsigned short* __restrict__ v_cache,
+    RopeArgs p) {
+  constexpr int HPW = 64 / LPH;                // heads per wave
+  extern __shared__ float cs_tab[];            // [half] cos, [half] sin
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub = lane % LPH;
+  const int half = p.half;
+  const float pos = (float)p.pos32[t];
+  for (int i = threadIdx.x; i < half; i += ROW_THREADS) {
+    float sn, cs;
+    sincosf(pos * p.inv_freq[i], &sn, &cs);
+    cs_tab[i] = cs * p.amp;
+    cs_tab[half + i] = sn * p.amp;
+  }
+  __syncthreads();
+  const int unit = (blockIdx.y * 4 + wave) * HPW + lane / LPH;
+  const bool active = unit < p.q_heads + p.k_heads;
+  const bool is_k = unit >= p.q_heads;
+  const int hd = is_k ? unit - p.q_heads : unit;
+  const int dim = !active ? 0 : is_k ? p.k_dim : p.q_dim;
+  const int nd = is_k ? p.k_nd : p.q_nd;
+  const int rot0 = is_k ? p.k_rot0 : p.q_rot0;
+  const float* w = is_k ? p.k_w : p.q_w;
+  const unsigned short* row = src + (long)t * p.ld_src +
+                              (is_k ? p.col_k : p.col_q) + (long)hd * dim;
+  float inv = 1.f;
+  {
+    // every lane walks the shuffles; heads without a norm add nothing
+    float ss = 0.f;
+    if (w != nullptr)
+      for (int c = sub * 8; c < min(nd, dim); c += LPH * 8) {
+        const u16x8 v = *reinterpret_cast<const u16x8*>(row + c);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) { const float f = bf2f(v[k]); ss += f * f; }
+      }
+#pragma unroll
+    for (int m = LPH / 2; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, WAVE_SIZE);
+    if (w != nullptr) inv = 1.0f / sqrtf(ss / (float)nd + p.eps);
+  }
+  if (!active) return;
+  long blk = 0;
+  int off = 0;
+  if (is_k) {
+    const long slot = p.slots[t];
+    if (slot < 0 || slot >= p.nslots) return;
+    blk = slot / p.BS;
+    off = (int)(slot % p.BS);
+  }
+  const int G = p.k_heads;
+  auto piece = [&](int c, float* f) {
+    const u16x8 v = *reinterpret_cast<const u16x8*>(row + c);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) f[k] = bf2f(v[k]);
+    if (w != nullptr && c < nd) {
+      const f32x4 w0 = *reinterpret_cast<const f32x4*>(w + c);
+      const f32x4 w1 = *reinterpret_cast<const f32x4*>(w + c + 4);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        f[k] = f[k] * inv * w0[k];
+        f[4 + k] = f[4 + k] * inv * w1[k];
+      }
+    }
+  };
+  for (int c = sub * 8; c < dim; c += LPH * 8) {
+    float f[8];
+    piece(c, f);
+    const int r = c - rot0;
+    if (rot0 >= 0 && r >= 0 && r < 2 * half) {
+      if (p.half_layout) {
+        const bool lower = r < half;
+        const int i0 = lower ? r : r - half;
+        float o[8];
+        piece(lower ? c + half : c - half, o);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const float cs = cs_tab[i0 + k], sn = cs_tab[half + i0 + k];
+          f[k] = lower ? f[k] * cs - o[k] * sn : f[k] * cs + o[k] * sn;
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < 8; k += 2) {
+          const int i = (r + k) >> 1;
+          const float cs = cs_tab[i], sn = cs_tab[half + i];
+          const float u2 = f[k] * cs - f[k + 1] * sn;
+          f[k + 1] = f[k + 1] * cs + f[k] * sn;
+          f[k] = u2;
+        }
+      }
+    }
+    u16x8 o8;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) o8[k] = f2bf(f[k]);
+    if (!is_k) {
+      *reinterpret_cast<u16x8*>(q_out + ((long)t * p.q_heads + hd) * dim + c) = o8;
+    } else {
+      *reinterpret_cast<u16x8*>(
+          k_cache + ((blk * G + hd) * p.BS + off) * (long)dim + c) = o8;
+      if (p.col_v < 0 && !p.skip_v && c < p.VW) {
+        unsigned short* dst =
+            v_cache + ((blk * G + hd) * (long)p.VW + c) * p.BS + off;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) dst[(long)k * p.BS] = o8[k];
+      }
+    }
+  }
+  if (is_k && p.col_v >= 0 && !p.skip_v) {
+    const unsigned short* vs = src + (long)t * p.ld_src + p.col_v + (long)hd * p.VW;
+    for (int c = sub * 8; c < p.VW; c += LPH * 8) {
+      const u16x8 v = *reinterpret_cast<const u16x8*>(vs + c);
+      unsigned short* dst =
+          v_cache + ((blk * G + hd) * (long)p.VW + c) * p.BS + off;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) dst[(long)k * p.BS] = v[k];
+    }
   }
 }
 
@@ -307,6 +435,37 @@ void head_rope_store_launch(void* q_out, const void* src, long ld_src,
   p.T = T;
   const dim3 grid(T, (q_heads + k_heads + 3) / 4);
   const size_t tab = (size_t)2 * half * sizeof(float);
+  auto m8 = [](long v) { return v % 8 == 0; };
+  const bool q_ok = q_heads == 0 ||
+      (m8(col_q) && m8(q_dim) && (q_w == nullptr || m8(q_nd)) &&
+       (q_rot0 < 0 || m8(q_rot0)) && (uintptr_t)q_out % 16 == 0);
+  const bool k_ok = k_heads == 0 ||
+      (m8(col_k) && m8(k_dim) && (k_w == nullptr || m8(k_nd)) &&
+       (k_rot0 < 0 || m8(k_rot0)) && m8(VW) && (col_v < 0 || m8(col_v)) &&
+       (uintptr_t)k_cache % 16 == 0);
+  if (bf && q_ok && k_ok && m8(ld_src) && (uintptr_t)src % 16 == 0 &&
+      (half == 0 || (half_layout ? m8(half) : m8(2 * half)))) {
+    const int widest = max(q_heads ? q_dim : 0, k_heads ? max(k_dim, VW) : 0);
+    int lph = 1;
+    while (lph < 64 && lph * 8 < widest) lph *= 2;
+    const int hpw = 64 / lph;
+    const dim3 vgrid(T, (q_heads + k_heads + 4 * hpw - 1) / (4 * hpw));
+#define HRS(L)                                                              \
+  head_rope_store_vec_kernel<L><<<vgrid, ROW_THREADS, tab, s>>>(            \
+      (unsigned short*)q_out, (const unsigned short*)src,                   \
+      (unsigned short*)k_cache, (unsigned short*)v_cache, p)
+    switch (lph) {
+      case 1: HRS(1); break;
+      case 2: HRS(2); break;
+      case 4: HRS(4); break;
+      case 8: HRS(8); break;
+      case 16: HRS(16); break;
+      case 32: HRS(32); break;
+      default: HRS(64); break;
+    }
+#undef HRS
+    return;
+  }
   if (bf)
     head_rope_store_kernel<unsigned short><<<grid, ROW_THREADS, tab, s>>>(
         (unsigned short*)q_out, (const unsigned short*)src,

@@ -448,7 +448,9 @@ __global__ __launch_bounds__(ROW_THREADS) void rotary_norm_store_vec_kernel(
 
 // Value rows of a prompt into the transposed value pages, a page at a
 // time. groups: int32 [n, 2] = first row, rows (<= 16) of runs that fall into
-// ONE page in order (host-built from the batch's sequences). A run that
+// ONE page in order (host-built from the batch's sequences). The source is
+// the projection (row = batch row) or, by_slot, a row-major pool (row =
+// slot). A run that
 // fills its whole page leaves as 16 keys per channel in one piece (32 bytes
 // of bf16 per lane, neighbouring lanes neighbouring channels); any other
 // run falls back to one store per (row, channel). CH channels at a time go
@@ -457,7 +459,7 @@ template <typename TS, int CH>
 __global__ __launch_bounds__(ROW_THREADS) void value_page_store_kernel(
     const TS* __restrict__ qkv, long ld_qkv, int v_col0,
     TS* __restrict__ v_cache, const long* __restrict__ slots, long nslots,
-    const int* __restrict__ groups, int T, int G, int VW) {
+    const int* __restrict__ groups, int T, int G, int VW, int by_slot) {
   constexpr int BS = 16;
   __shared__ TS tile[BS][CH + 8];
   __shared__ long s_slot[BS];
@@ -476,7 +478,11 @@ __global__ __launch_bounds__(ROW_THREADS) void value_page_store_kernel(
     __syncthreads();
     for (int i = tid; i < nrows * cw; i += ROW_THREADS) {
       const int r = i / cw, c = i % cw;
-      tile[r][c] = qkv[(long)(row0 + r) * ld_qkv + v_col0 + c0 + c];
+      // by_slot: the source is a row-major pool indexed like the slots (a
+      // key pool whose rows' first channels are the values)
+      long srow = row0 + r;
+      if (by_slot) srow = min(max(s_slot[r], 0L), nslots - 1);
+      tile[r][c] = qkv[srow * ld_qkv + v_col0 + c0 + c];
     }
     __syncthreads();
     if (fast) {
@@ -679,16 +685,16 @@ void rotary_norm_store_launch(void* q_out, const void* qkv, long ld_qkv, int nq,
 void value_page_store_launch(const void* qkv, long ld_qkv, int v_col0,
                              void* v_cache, const long* slots, long nslots,
                              const int* groups, int ngroups, int T, int G,
-                             int VW, int bf, hipStream_t s) {
+                             int VW, int bf, int by_slot, hipStream_t s) {
   if (ngroups <= 0) return;
   if (bf)
     value_page_store_kernel<unsigned short, 1024><<<ngroups, ROW_THREADS, 0, s>>>(
         (const unsigned short*)qkv, ld_qkv, v_col0, (unsigned short*)v_cache,
-        slots, nslots, groups, T, G, VW);
+        slots, nslots, groups, T, G, VW, by_slot);
   else
     value_page_store_kernel<float, 512><<<ngroups, ROW_THREADS, 0, s>>>(
         (const float*)qkv, ld_qkv, v_col0, (float*)v_cache, slots, nslots,
-        groups, T, G, VW);
+        groups, T, G, VW, by_slot);
 }
 
 void diff_combine_launch(void* out, const float* a, const float* lam,

@@ -11,7 +11,7 @@
 void embed_rows_scaled_launch(float*, const long*, const void*, int, int, long, float, int, hipStream_t);
 void add_layer_norm_launch(float*, const void*, const float*, const float*, void*, int, int, float, int, int, hipStream_t);
 void head_norm_store_launch(void*, void*, long, int, int, int, const float*, const float*, int, float, float, const int*, const void*, long, const float*, void*, void*, const long*, long, int, int, int, float, int, int, int, hipStream_t);
-void value_page_store_launch(const void*, long, int, void*, const long*, long, const int*, int, int, int, int, int, hipStream_t);
+void value_page_store_launch(const void*, long, int, void*, const long*, long, const int*, int, int, int, int, int, int, hipStream_t);
 void route_topk_launch(int*, float*, const float*, int, const float*, int, int, int, int, int, int, int, int, float, hipStream_t);
 void causal_conv_silu_launch(void*, const void*, long, int, int, int, const float*, const float*, void*, const int*, const int*, const int*, const int*, const int*, int, int, int, int, hipStream_t);
 int state_scan_launch(float*, const void*, long, int, int, int, const void*, long, int, int, int, int, int, int, const float*, const float*, const float*, const float*, float*, const int*, const int*, const int*, const int*, int, int, int, int, int, hipStream_t);
@@ -163,7 +163,7 @@ void head_norm_store(Tensor q_out, Tensor qkv, long nq, long nk, Tensor q_w,
                             v_cache.data_ptr(), slots.data_ptr<long>(),
                             k_cache.size(0) * (long)BS,
                             page_groups->data_ptr<int>(),
-                            (int)page_groups->size(0), T, G, VW, bf,
+                            (int)page_groups->size(0), T, G, VW, bf, 0,
                             cur_stream(qkv));
     HIP_CHECK_LAST();
   }

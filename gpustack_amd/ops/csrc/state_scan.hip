@@ -607,6 +607,50 @@ __global__ __launch_bounds__(ROW_THREADS) void gated_group_norm_vec_kernel(
   }
 }
 
+// bf16 gates and outputs, parts of a multiple of 4 and at most 256
+// channels (per-head norms): LPG lanes share a part, 4 channels each in one
+// step, a wave takes 64 / LPG parts of a row and a workgroup four times that.
+template <int LPG>
+__global__ __launch_bounds__(ROW_THREADS) void gated_group_norm_small_kernel(
+    unsigned short* __restrict__ out, const float* __restrict__ y,
+    const unsigned short* __restrict__ gate, long ld_gate,
+    const float* __restrict__ w, int C, int gs, int groups, float eps,
+    int gate_first) {
+  constexpr int GPW = 64 / LPG;
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int grp = (blockIdx.y * 4 + wave) * GPW + lane / LPG;
+  const int c = (lane % LPG) * 4;
+  const bool live = grp < groups && c < gs;
+  const int c0 = grp * gs + c;
+  float u[4] = {0.f, 0.f, 0.f, 0.f}, gv[4] = {0.f, 0.f, 0.f, 0.f};
+  float ss = 0.f;
+  if (live) {
+    const f32x4 yv = *reinterpret_cast<const f32x4*>(y + t * C + c0);
+    const u16x4 g4 = *reinterpret_cast<const u16x4*>(gate + t * ld_gate + c0);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      gv[k] = bf2f(g4[k]);
+      u[k] = gate_first == 1 ? yv[k] * silu_f(gv[k]) : yv[k];
+      ss += u[k] * u[k];
+    }
+  }
+#pragma unroll
+  for (int m = LPG / 2; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, WAVE_SIZE);
+  if (!live) return;
+  const float inv = 1.0f / sqrtf(ss / (float)gs + eps);
+  const f32x4 wv = *reinterpret_cast<const f32x4*>(w + c0);
+  u16x4 o;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    float r = u[k] * inv * wv[k];
+    if (gate_first == 0) r *= sigmoid_f(gv[k]);
+    else if (gate_first == 2) r *= silu_f(gv[k]);
+    o[k] = f2bf(r);
+  }
+  *reinterpret_cast<u16x4*>(out + t * C + c0) = o;
+}
+
 template <typename TS, typename TD, int NR, int TPP>
 void scan_launch(float* y, const void* src, const void* dt, const ScanArgs& p,
                  int nseq, hipStream_t s) {
@@ -753,6 +797,28 @@ void gated_group_norm_launch(void* out, const float* y, const void* gate,
   if (T <= 0) return;
   dim3 grid(T, groups);
   const int gs = C / groups;
+  if (gate_bf && out_bf && gs % 4 == 0 && C % 4 == 0 && ld_gate % 4 == 0 &&
+      gs <= 256 && groups > 1 && ((uintptr_t)gate % 8) == 0) {
+    int lpg = 1;
+    while (lpg * 4 < gs) lpg *= 2;
+    const int gpb = 4 * (64 / lpg);
+    const dim3 sgrid(T, (groups + gpb - 1) / gpb);
+#define GGN(L)                                                               \
+  gated_group_norm_small_kernel<L><<<sgrid, ROW_THREADS, 0, s>>>(            \
+      (unsigned short*)out, y, (const unsigned short*)gate, ld_gate, w, C,   \
+      gs, groups, eps, gate_first)
+    switch (lpg) {
+      case 1: GGN(1); break;
+      case 2: GGN(2); break;
+      case 4: GGN(4); break;
+      case 8: GGN(8); break;
+      case 16: GGN(16); break;
+      case 32: GGN(32); break;
+      default: GGN(64); break;
+    }
+#undef GGN
+    return;
+  }
   if (gate_bf && out_bf && gs % 4 == 0 && C % 4 == 0 && ld_gate % 4 == 0 &&
       gs <= 4096 && ((uintptr_t)gate % 8) == 0) {
     if (gs <= 1024)

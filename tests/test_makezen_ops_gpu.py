@@ -128,6 +128,28 @@ def test_head_rope_store_values_by_page(dtype):
     for a, b, nm in zip(run("cuda", groups), ref, "qkv"):
         close(a, b, dtype, nm)
 
+    # a latent row: the values are the finished key row's first channels
+    # and leave page by page out of the key pool
+    QR, R, RD = 24, 48, 8
+    src2 = torch.randn(T, QR + R + RD, generator=g).to(dtype)
+    wq, wr = torch.rand(QR, generator=g) + 0.5, torch.rand(R, generator=g) + 0.5
+
+    def run_latent(dev, pg=None):
+        to = lambda t: t.to(dev)
+        cq = torch.zeros(T, QR, dtype=dtype, device=dev)
+        kc = torch.zeros(6, 1, BS, R + RD, dtype=dtype, device=dev)
+        vc = torch.zeros(6, 1, R, BS, dtype=dtype, device=dev)
+        fn = ops.head_rope_store if dev == "cuda" else torch_ref.head_rope_store
+        kw_ = {"page_groups": pg} if dev == "cuda" else {}
+        fn(cq, to(src2), 0, 1, QR, to(wq), QR, -1, QR, 1, R + RD, to(wr), R, R,
+           -1, to(invf), True, 1.2, to(pos), kc, vc, to(slots), eps, **kw_)
+        return cq, kc, vc
+
+    ref = run_latent("cpu")
+    for pg in (None, groups):
+        for a, b, nm in zip(run_latent("cuda", pg), ref, "qkv"):
+            close(a, b, dtype, "latent " + nm)
+
 
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("H,G,N,P", [(4, 2, 6, 5), (2, 2, 16, 8), (3, 1, 5, 12),
