@@ -141,8 +141,11 @@ def attend(q, k, v, scale, window=0, sink=None, softcap=0.0):
     s = (q @ k.t()) * scale
     if softcap:
         s = softcap * torch.tanh(s / softcap)
-    mask = torch.tensor([[visible(i, j, window) for j in range(T)]
-                         for i in range(T)])
+    i, j = torch.arange(T)[:, None], torch.arange(T)[None, :]
+    mask = (j <= i) & ((i - j < window) if window > 0 else (j <= i))
+    if T <= 8:      # the table above is `visible`, element by element
+        assert all(bool(mask[a, b]) == visible(a, b, window)
+                   for a in range(T) for b in range(T))
     s = s.masked_fill(~mask, -float("inf"))
     mx = s.max(-1, keepdim=True)[0]
     if sink is not None:
