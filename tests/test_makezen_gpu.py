@@ -171,6 +171,28 @@ def test_long_decoding_fp32(tmp_path, gpu_engine):
     assert tf.err(got, oracle.forward(cfg, w, toks)) < 5e-4
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_context_with_key_split(tmp_path, gpu_engine, dtype):
+    """A context long enough for the attention kernels to split a decode
+    row's keys over workgroups (MFMA path), behind a window of 600, with
+    sinks, on latent rows and on capped softmax heads."""
+    import copy
+
+    kw = dict(ALIGNED, layers=copy.deepcopy(ALIGNED["layers"]))
+    kw["layers"][0]["mixer"]["mask"]["size"] = 600
+    kw["layers"][3]["mixer"]["mask"]["size"] = 530
+    cfg, w, d = _model(tmp_path, kw)
+    toks = tf.tokens_for(cfg, 650, 21)
+    steps = [[("a", 300)], [("a", 340)]] + [[("a", 1)]] * 10
+    ref = oracle.forward(cfg, w, toks)
+    got = tf.replay(gpu_engine(d, dtype=dtype, blocks=60), {"a": toks},
+                    steps)["a"]
+    if dtype == "float32":
+        assert tf.err(got, ref) < 5e-4
+    else:
+        assert rows_over(got, ref, 0.15) <= 0.1
+
+
 @pytest.mark.parametrize("kind", ["latent", "softmax"])
 @pytest.mark.parametrize("far_pos", [0, 16, 511, 700])
 @pytest.mark.parametrize("decode", [False, True])
