@@ -152,6 +152,14 @@ def test_other_sizes_fp32_and_bf16(tmp_path, gpu_engine):
                             q_rank=9, window=500, scaling=False),
         oracle.latent_layer(heads=2, dim=5, rot_dim=6, vdim=2, kv_rank=7,
                             q_rank=4, window=3, kv_from=3, scaling=False),
+        # more heads on one key stream than a workgroup's tile holds
+        oracle.latent_layer(heads=20, dim=2, rot_dim=4, vdim=3, kv_rank=6,
+                            q_rank=5, window=9, ff=0),
+        oracle.parallel_layer(
+            left=oracle.softmax_entry(heads=36, kv_heads=2, dim=4, vdim=2,
+                                      rot_dims=4),
+            right=oracle.delta_mixer_entry(heads=2, kv_heads=1, dim=4, vdim=4,
+                                           conv=2), ff=0),
     ]
     cfg, w, d = _model(tmp_path, dict(width=18, layers=layers))
     toks = tf.tokens_for(cfg, 37, 11)
